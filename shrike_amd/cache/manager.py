@@ -6,8 +6,9 @@ Layers whose mixers ask for the same PagedSpec form a group; a group has its
 own pool of pages, its own device tensors (whatever the spec lists per page,
 each as ``[layers, pages + 1, *its shape for one page]``: what a page holds and
 how it is laid out is the mixer's business, not the manager's) and, per request,
-its own block table.  A group with a window gives pages back as soon as no later
-query can reach them (table entry -1); all pages come back when the request ends.
+its own block table.  A group with a window or a block-local mask gives pages back
+as soon as no later query can reach them (table entry -1); all pages come back when
+the request ends.
 Layers whose mixers ask for a StateSpec form state groups: a tensor
 ``[layers, slots, *shape]`` indexed by the request's state slot.  Every request
 holds one slot, whether or not any layer has state.
@@ -109,7 +110,7 @@ class CacheManager:
         self.enable_prefix_caching = bool(
             enable_prefix_caching
             and not self.state_groups
-            and all(g.spec.window is None for g in self.groups)
+            and all(not g.spec.bounded for g in self.groups)
         )
         self.cache_hit_blocks = 0
         self.cache_query_blocks = 0
@@ -201,18 +202,21 @@ class CacheManager:
                 table.append(g.pool.take())
 
     def trim(self, seq: SequenceCache, num_computed: int) -> int:
-        """Give back the pages of windowed groups that no later query can reach.
+        """Give back the pages of groups with a window or a block-local mask that no
+        later query can reach.
 
         After `num_computed` tokens the next query sits at position >=
-        num_computed and reads keys > num_computed - window; pages that end at
-        or before num_computed - window + 1 are done.  Returns pages released.
+        num_computed.  With a window it reads keys > num_computed - window; with
+        blocks of `chunk` positions, keys from the start of num_computed's block on
+        (a later query's first key is no older: neither bound falls as positions
+        rise).  Pages that end at or before that first key are done.  Returns pages
+        released.
         """
         released = 0
         for gi, (g, table) in enumerate(zip(self.groups, seq.tables)):
-            w = g.spec.window
-            if w is None:
+            if not g.spec.bounded:
                 continue
-            first_needed = max(0, num_computed - w + 1)
+            first_needed = g.spec.first_needed(num_computed)
             done = min(first_needed // self.page_size, len(table))
             for i in range(seq._trimmed[gi], done):
                 if table[i] >= 0:

@@ -106,11 +106,13 @@ def architecture_name(raw: dict) -> str:
     archs = raw.get("architectures")
     if isinstance(archs, (list, tuple)) and archs:
         return str(archs[0])
+    if isinstance(raw.get("architecture"), str):  # some formats name one, as a string
+        return raw["architecture"]
     mt = raw.get("model_type")
     if mt in _MODEL_TYPES:
         return _MODEL_TYPES[mt]
     raise ConfigError(
-        "config.json names no architecture: expected \"architectures\": [name] "
+        "config.json names no architecture: expected \"architectures\": [name] or \"architecture\": name "
         f"(registered: {', '.join(architectures())})"
     )
 

@@ -12,13 +12,22 @@ from __future__ import annotations
 from dataclasses import dataclass, field
 from typing import ClassVar
 
+# Every part finds its tensors under its own name plus a sub-name per role ("weight",
+# "q_proj.weight", ...).  A spec's `names` replaces those sub-names for architectures whose
+# files spell them otherwise: pairs (role, sub-name); an empty sub-name stands for the
+# part's own name.
+Names = tuple
+
 
 @dataclass(frozen=True)
 class RMSNormSpec:
-    """y = x * rsqrt(mean(x^2) + eps) * weight."""
+    """y = x * rsqrt(mean(x^2) + eps) * (offset + weight): offset 0 for a weight that is
+    stored as it is applied, 1 for one that is stored around zero."""
 
     kind: ClassVar[str] = "rmsnorm"
     eps: float
+    offset: float = 0.0
+    names: Names = ()
 
 
 @dataclass(frozen=True)
@@ -31,12 +40,26 @@ class RotarySpec:
 
 
 @dataclass(frozen=True)
+class RotaryAdjacentSpec:
+    """Rotation of neighbouring elements (2i, 2i + 1), i < rotary_dim / 2, by
+    position * theta**(-2i/rotary_dim); elements from rotary_dim on stay as they are."""
+
+    kind: ClassVar[str] = "rotary_adjacent"
+    theta: float
+    rotary_dim: int
+
+
+@dataclass(frozen=True)
 class AttentionSpec:
     """Causal grouped-query attention over a paged key/value cache.
 
     ``window``: a query at position p reads keys j with p - window < j <= p;
-    None reads every key.  ``position`` is applied to queries and keys after
-    the projections; None leaves them as they are.
+    None reads every key.  ``chunk``: a query reads only the keys j <= p of its own
+    block of `chunk` positions, floor(j / chunk) == floor(p / chunk), blocks counted
+    from position 0 of the sequence; None sets no such bound.  ``position`` is
+    applied to queries and keys after the projections; None leaves them as they
+    are.  ``values_from_keys``: there is no value projection; a token's values are
+    its keys as projected, before ``position`` is applied.
     """
 
     kind: ClassVar[str] = "paged_attention"
@@ -47,7 +70,10 @@ class AttentionSpec:
     out_bias: bool
     scale: float
     window: int | None = None
-    position: RotarySpec | None = None
+    position: object = None
+    chunk: int | None = None
+    values_from_keys: bool = False
+    names: Names = ()
 
 
 @dataclass(frozen=True)
@@ -58,6 +84,25 @@ class SwiGLUSpec:
     kind: ClassVar[str] = "swiglu"
     intermediate_size: int
     activation: str = "silu"
+    names: Names = ()
+
+
+@dataclass(frozen=True)
+class TokenSideSpec:
+    """A second input per token and layer, gated by the stream:
+    y = proj(act(gate(x)) * table[token, index*dim : (index+1)*dim]);
+    x += y * rsqrt(mean(y^2) + eps) * weight.  ``table_name`` is the full name of the
+    table [vocab, slices * dim], which all layers share."""
+
+    kind: ClassVar[str] = "token_side"
+    vocab_size: int
+    dim: int
+    index: int
+    slices: int
+    eps: float
+    activation: str = "gelu_tanh"
+    table_name: str = "side.embed"
+    names: Names = ()
 
 
 @dataclass(frozen=True)
@@ -81,11 +126,30 @@ class BlockSpec:
 
 
 @dataclass(frozen=True)
+class ParallelBlockSpec:
+    """h = norm(x); x += mixer(h) + ffn(h); then x = side(x, tokens) where there is one.
+    One norm feeds both sublayers; ``ffn`` and ``side`` may be None."""
+
+    kind: ClassVar[str] = "parallel_residual"
+    name: str
+    norm: object
+    mixer: object
+    ffn: object = None
+    side: object = None
+    norm_name: str = "norm1"
+    mixer_name: str = "mix"
+    ffn_name: str = "mlp"
+    side_name: str = "side"
+
+
+@dataclass(frozen=True)
 class TokenEmbeddingSpec:
-    """x = table[token id], no scaling."""
+    """x = table[token id] * scale."""
 
     kind: ClassVar[str] = "token_lookup"
     vocab_size: int
+    scale: float = 1.0
+    names: Names = ()
 
 
 @dataclass(frozen=True)
@@ -94,15 +158,21 @@ class LinearHeadSpec:
 
     kind: ClassVar[str] = "linear"
     vocab_size: int
+    names: Names = ()
 
 
 @dataclass(frozen=True)
 class ScheduleEntry:
     """One run of a block.  ``cache_of`` names an earlier schedule position whose
-    cache this run reads instead of owning one; None means it owns its cache."""
+    cache this run reads instead of owning one; None means it owns its cache.
+    Before the run, ``add_embedding`` adds the embedding's output (the stream as it
+    was before the first block) to the stream, and ``add_vector`` = (tensor, row)
+    adds row `row` of a tensor that the model declares in ``stream_vectors``."""
 
     block: int
     cache_of: int | None = None
+    add_embedding: bool = False
+    add_vector: tuple | None = None
 
 
 @dataclass(frozen=True)
@@ -129,6 +199,9 @@ class ModelSpec:
     extra: dict = field(default_factory=dict, compare=False)
     embedding: object = None
     head: object = None
+    # (tensor name, rows): float32 tensors [rows, hidden_size] whose rows schedule
+    # entries add to the stream (ScheduleEntry.add_vector)
+    stream_vectors: tuple = ()
 
     def __post_init__(self):
         if self.embedding is None:
@@ -142,6 +215,10 @@ class ModelSpec:
         for pos, entry in enumerate(self.schedule):
             if not 0 <= entry.block < len(self.blocks):
                 raise ValueError(f"schedule[{pos}] names block {entry.block}, which does not exist")
+            if entry.add_vector is not None:
+                rows = dict(self.stream_vectors).get(entry.add_vector[0])
+                if rows is None or not 0 <= entry.add_vector[1] < rows:
+                    raise ValueError(f"schedule[{pos}] adds {entry.add_vector}, which stream_vectors does not hold")
             if entry.cache_of is not None:
                 if not 0 <= entry.cache_of < pos:
                     raise ValueError(

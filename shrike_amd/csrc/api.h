@@ -31,9 +31,33 @@ int shk_gather_rows(const int32_t* src, long long ld, int src_rows, const int32_
 // it may be recorded into a HIP graph).
 int shk_zero_bytes(void* dst, long long bytes, void* stream);
 
-// out[i, :] = float(table[ids[i], :]); ids must lie in [0, vocab).
+// out[i, :] = float(table[ids[i], :]) * scale; ids must lie in [0, vocab).
 int shk_embed(const void* table, int dtype, const int32_t* ids, float* out, int n, int hidden,
-              int vocab, void* stream);
+              int vocab, float scale, void* stream);
+
+// resid[r, :] += other[r, :] + vec[:] for r < n (float32; other and vec may be null).
+int shk_add_rows(float* resid, const float* other, const float* vec, int n, int hidden, void* stream);
+
+// resid[r, :] += d1[r, :] + d2[r, :], and cast[r, :] = the new resid[r, :] in `dtype`
+// (d2 and cast may be null).  d1 and d2 are outputs of products: tensors of `dtype`
+// (splits 0) or float32 partial sums [splits][n][hidden], added in order.
+int shk_add_deltas(float* resid, const void* d1, int splits1, const void* d2, int splits2, void* cast,
+                   int dtype, int n, int hidden, void* stream);
+
+// A product's output that is normed by itself before it joins the stream:
+// x = resid[row] + delta[row] * rsqrt(mean(delta[row]^2) + deps) * dweight, stored back
+// with write_resid; with out != null, out[r] = x * rsqrt(mean(x^2) + eps) * weight as
+// well (the norm that follows).  delta / delta_splits / rows / resid_rows as in
+// shk_add_rmsnorm, except that delta has `dtype` or is float32 partial sums.
+int shk_add_normed_rmsnorm(float* resid, const void* delta, int delta_splits, const float* dweight,
+                           float deps, const float* weight, float eps, void* out, int dtype,
+                           const int32_t* rows, int n, int hidden, int write_resid, int resid_rows,
+                           void* stream);
+
+// out[r, j] = act(a[r, j]) * table[ids[r] * ld + offset + j] for j < width: a gate times
+// a slice of the table row that the token chooses.  ids must lie in [0, table_rows).
+int shk_act_mul_rows(const void* a, const void* table, int dtype, const int32_t* ids, long long ld,
+                     int offset, int table_rows, void* out, int n, int width, int act, void* stream);
 
 // Residual add fused with RMSNorm.  For each of n rows r (row index rows[r]
 // when `rows` is given, else r):  x = resid[row] (+ delta[row]);  if
@@ -104,20 +128,26 @@ int shk_mfma_alone(const void* operands, float* out, int workgroups, int iters, 
 // [splits][n][width] of a product split along k; they are added in order, `bias`
 // (float32 [width] or null) is added, and the rotated queries are written to
 // qkv's query columns (qkv is then output only).
+// pairing 1 pairs the neighbours (2i, 2i + 1) instead, with the same angle for pair i.
+// v_from_k != 0: there are no value columns, qkv is [n, (heads + kv_heads) * head_dim],
+// and a token's values are its keys as they were projected, before the rotation.
 int shk_rope_kv_store(void* qkv, int dtype, int n, int heads, int kv_heads, int head_dim,
                       int rot_dim, const float* inv_freq, const int32_t* positions,
                       const int32_t* token_seq, const int32_t* tables, int table_stride,
                       void* k_pool, void* v_pool, int page_size, int num_pages, int write_kv,
-                      const float* parts, int splits, const float* bias, void* stream);
+                      const float* parts, int splits, const float* bias, int pairing,
+                      int v_from_k, void* stream);
 
 // Causal attention of n query tokens over their sequences' paged caches.
 // Token t (position p, sequence s) reads keys j in (p - window, p] (all j <= p
-// when window <= 0) through tables[s].  q has row stride q_stride elements,
+// when window <= 0) through tables[s]; with chunk > 0 only those of them that lie
+// in p's own block of `chunk` positions, floor(j / chunk) == floor(p / chunk) (the
+// same two bounds in every attention launcher below).  q has row stride q_stride elements,
 // out is [n, heads * head_dim].  Softmax and accumulation are float32.
 int shk_attention(const void* q, int q_stride, void* out, int dtype, int n, int heads,
                   int kv_heads, int head_dim, const int32_t* positions, const int32_t* token_seq,
                   const int32_t* tables, int table_stride, int num_seqs, const void* k_pool,
-                  const void* v_pool, int page_size, int num_pages, int window, float scale,
+                  const void* v_pool, int page_size, int num_pages, int window, int chunk, float scale,
                   void* stream);
 
 // 1 if the MFMA attention kernels take these shapes (head_dim a multiple of 32
@@ -133,7 +163,7 @@ int shk_attention_supports_mfma(int heads, int kv_heads, int head_dim, int page_
 int shk_attention_decode_bf16(const void* q, int q_stride, void* out, int num_seqs, int heads,
                               int kv_heads, int head_dim, const int32_t* positions,
                               const int32_t* tables, int table_stride, const void* k_pool,
-                              const void* v_pool, int page_size, int window, float scale,
+                              const void* v_pool, int page_size, int window, int chunk, float scale,
                               float* partial, int nsplit, int streaming, void* stream);
 
 // bfloat16 attention for prompt portions, in tiles of 16 queries: tile i covers
@@ -143,7 +173,7 @@ int shk_attention_prefill_bf16(const void* q, int q_stride, void* out, int num_t
                                int kv_heads, int head_dim, const int32_t* cu_q,
                                const int32_t* ctx_lens, const int32_t* tile_seq,
                                const int32_t* tile_q0, const int32_t* tables, int table_stride,
-                               const void* k_pool, const void* v_pool, int page_size, int window,
+                               const void* k_pool, const void* v_pool, int page_size, int window, int chunk,
                                float scale, void* stream);
 
 // The same for all query heads of a key/value head at once: a workgroup serves
@@ -165,7 +195,7 @@ int shk_attention_prefill_shared_bf16(const void* q, int q_stride, void* out, in
                                       const int32_t* ctx_lens, const int32_t* wg_seq,
                                       const int32_t* wg_q0, const int32_t* tables,
                                       int table_stride, const void* k_pool, const void* v_pool,
-                                      int page_size, int window, float scale, int small,
+                                      int page_size, int window, int chunk, float scale, int small,
                                       float* partial, int nsplit, int first_token,
                                       int prompt_tokens, void* stream);
 

@@ -23,7 +23,7 @@ __global__ void __launch_bounds__(kAttnThreads)
                              const int32_t* __restrict__ token_seq,
                              const int32_t* __restrict__ tables, int table_stride,
                              const T* __restrict__ k_pool, const T* __restrict__ v_pool,
-                             int page_size, int num_pages, int window, float scale) {
+                             int page_size, int num_pages, int window, int chunk, float scale) {
   __shared__ float qs[kMaxHeadDim];
   __shared__ float probs[kAttnThreads];
   __shared__ int32_t rows[kAttnThreads];  // key-cache row of each key of the tile, -1 if masked
@@ -34,7 +34,7 @@ __global__ void __launch_bounds__(kAttnThreads)
   const int kvh = head / (heads / kv_heads);
   const int pos = positions[t];
   const int32_t* table = tables + static_cast<size_t>(token_seq[t]) * table_stride;
-  const int lo = (window > 0 && pos - window + 1 > 0) ? pos - window + 1 : 0;
+  const int lo = first_key(pos, window, chunk);
 
   const T* qrow = q + static_cast<size_t>(t) * q_stride + head * head_dim;
   for (int d = threadIdx.x; d < head_dim; d += kAttnThreads) qs[d] = to_float(qrow[d]);
@@ -108,7 +108,7 @@ extern "C" int shk_attention(const void* q, int q_stride, void* out, int dtype, 
                              int kv_heads, int head_dim, const int32_t* positions,
                              const int32_t* token_seq, const int32_t* tables, int table_stride,
                              int num_seqs, const void* k_pool, const void* v_pool, int page_size,
-                             int num_pages, int window, float scale, void* stream) {
+                             int num_pages, int window, int chunk, float scale, void* stream) {
   SHK_REQUIRE(dtype == kF32 || dtype == kBF16, "attention: unknown dtype %d", dtype);
   SHK_REQUIRE(n >= 0 && heads > 0 && kv_heads > 0 && heads % kv_heads == 0,
               "attention: heads=%d must be a positive multiple of kv_heads=%d", heads, kv_heads);
@@ -131,12 +131,12 @@ extern "C" int shk_attention(const void* q, int q_stride, void* out, int dtype, 
     attention_generic_kernel<float><<<grid, kAttnThreads, 0, s>>>(
         static_cast<const float*>(q), q_stride, static_cast<float*>(out), heads, kv_heads, head_dim,
         positions, token_seq, tables, table_stride, static_cast<const float*>(k_pool),
-        static_cast<const float*>(v_pool), page_size, num_pages, window, scale);
+        static_cast<const float*>(v_pool), page_size, num_pages, window, chunk, scale);
   else
     attention_generic_kernel<bf16><<<grid, kAttnThreads, 0, s>>>(
         static_cast<const bf16*>(q), q_stride, static_cast<bf16*>(out), heads, kv_heads, head_dim,
         positions, token_seq, tables, table_stride, static_cast<const bf16*>(k_pool),
-        static_cast<const bf16*>(v_pool), page_size, num_pages, window, scale);
+        static_cast<const bf16*>(v_pool), page_size, num_pages, window, chunk, scale);
   SHK_LAUNCH_CHECK("attention");
   return 0;
 }

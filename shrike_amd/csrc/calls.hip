@@ -60,6 +60,10 @@ const Launcher kLaunchers[] = {
     SHK_LAUNCHER(shk_embed),
     SHK_LAUNCHER(shk_add_rmsnorm),
     SHK_LAUNCHER(shk_act_mul),
+    SHK_LAUNCHER(shk_add_rows),
+    SHK_LAUNCHER(shk_add_deltas),
+    SHK_LAUNCHER(shk_add_normed_rmsnorm),
+    SHK_LAUNCHER(shk_act_mul_rows),
     SHK_LAUNCHER(shk_gemm),
     SHK_LAUNCHER(shk_gemm_bf16_tiled_weight),
     SHK_LAUNCHER(shk_rope_kv_store),

@@ -91,6 +91,20 @@ __host__ __device__ inline size_t key_offset(int slot, int d, int page_size, int
   return (static_cast<size_t>(d / slab) * page_size + slot) * slab + d % slab;
 }
 
+// ------------------------------------------------------- which keys a query reads
+// The first key that the query at position `pos` reads; its last is `pos` itself.
+// window > 0: only the last `window` keys.  chunk > 0: only keys of the query's own
+// block of `chunk` positions, blocks counted from position 0 of the sequence.  Both
+// bounds may hold at once; neither falls as the position rises.
+__host__ __device__ inline int first_key(int pos, int window, int chunk) {
+  int lo = (window > 0 && pos - window + 1 > 0) ? pos - window + 1 : 0;
+  if (chunk > 0 && pos > 0) {
+    const int block = pos / chunk * chunk;
+    lo = block > lo ? block : lo;
+  }
+  return lo;
+}
+
 // ---------------------------------------------------------------- host side
 
 enum DType : int { kF32 = 0, kBF16 = 1 };

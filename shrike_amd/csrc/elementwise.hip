@@ -21,11 +21,11 @@ void set_error(const char* fmt, ...) {
 
 template <typename T>
 __global__ void embed_kernel(const T* __restrict__ table, const int32_t* __restrict__ ids,
-                             float* __restrict__ out, int hidden) {
+                             float* __restrict__ out, int hidden, float scale) {
   const int row = blockIdx.x;
   const T* src = table + static_cast<size_t>(ids[row]) * hidden;
   float* dst = out + static_cast<size_t>(row) * hidden;
-  for (int i = threadIdx.x; i < hidden; i += blockDim.x) dst[i] = to_float(src[i]);
+  for (int i = threadIdx.x; i < hidden; i += blockDim.x) dst[i] = to_float(src[i]) * scale;
 }
 
 // ------------------------------------------------------------ add + RMSNorm
@@ -161,6 +161,181 @@ __global__ void act_mul_kernel(const T* __restrict__ gu, T* __restrict__ out, in
   out[row * inter + j] = from_float<T>(s * u);
 }
 
+// ------------------------------------------------- rows held in registers
+// The kernels below keep one row per workgroup in registers: V elements per access
+// (4: whole vectors, for widths that are a multiple of 4 and aligned buffers; 1:
+// every other width), kRowSlots accesses per thread, THREADS threads.
+
+constexpr int kRowSlots = 8;
+
+template <int V>
+struct RowVec {
+  float v[V];
+};
+
+template <int V, typename T>
+__device__ __forceinline__ RowVec<V> row_load(const T* p) {
+  RowVec<V> r;
+  if constexpr (V == 4) {
+    const float4 f = load4(p);
+    r.v[0] = f.x, r.v[1] = f.y, r.v[2] = f.z, r.v[3] = f.w;
+  } else {
+    r.v[0] = to_float(p[0]);
+  }
+  return r;
+}
+
+template <int V, typename T>
+__device__ __forceinline__ void row_store(T* p, const RowVec<V>& r) {
+  if constexpr (V == 4) {
+    store4(p, make_float4(r.v[0], r.v[1], r.v[2], r.v[3]));
+  } else {
+    p[0] = from_float<T>(r.v[0]);
+  }
+}
+
+// The sum of a product's output for one row: a tensor of T (splits 0) or the float32
+// partial sums [splits][rows][hidden] of a product split along k, added in order.
+template <int V, int THREADS, typename T>
+__device__ __forceinline__ void row_gather(const void* delta, int splits, size_t split_stride,
+                                           size_t row, int hidden, RowVec<V> (&d)[kRowSlots]) {
+  const int nvec = hidden / V;
+#pragma unroll
+  for (int i = 0; i < kRowSlots; ++i) {
+    const int c = threadIdx.x + i * THREADS;
+#pragma unroll
+    for (int e = 0; e < V; ++e) d[i].v[e] = 0.f;
+    if (c >= nvec) continue;
+    if (splits == 0) {
+      d[i] = row_load<V>(static_cast<const T*>(delta) + row * hidden + c * V);
+    } else {
+      const float* p = static_cast<const float*>(delta) + row * hidden + c * V;
+      for (int z = 0; z < splits; ++z) {
+        const RowVec<V> more = row_load<V>(p + z * split_stride);
+#pragma unroll
+        for (int e = 0; e < V; ++e) d[i].v[e] += more.v[e];
+      }
+    }
+  }
+}
+
+// resid[r] += other[r] + vec: a second stream and a vector that is the same for every row
+// (either may be absent).
+__global__ void __launch_bounds__(256)
+    add_rows_kernel(float* __restrict__ resid, const float* __restrict__ other,
+                    const float* __restrict__ vec, int hidden) {
+  const size_t base = static_cast<size_t>(blockIdx.x) * hidden;
+  for (int i = threadIdx.x; i < hidden; i += 256) {
+    float v = resid[base + i];
+    if (other) v += other[base + i];
+    if (vec) v += vec[i];
+    resid[base + i] = v;
+  }
+}
+
+// resid[r] += d1[r] + d2[r]; cast[r] = T(resid[r]).  d1 and d2 are outputs of products
+// (see row_gather); d2 and cast may be absent.  (d1 + d2) is formed first, then added.
+template <typename T, int V, int THREADS>
+__global__ void __launch_bounds__(THREADS)
+    add_deltas_kernel(float* __restrict__ resid, const void* __restrict__ d1, int splits1,
+                      const void* __restrict__ d2, int splits2, T* __restrict__ cast, int hidden,
+                      size_t split_stride) {
+  const size_t row = blockIdx.x;
+  const int nvec = hidden / V;
+  RowVec<V> a[kRowSlots], b[kRowSlots], x[kRowSlots];
+#pragma unroll
+  for (int i = 0; i < kRowSlots; ++i) {
+    const int c = threadIdx.x + i * THREADS;
+    if (c < nvec) x[i] = row_load<V>(resid + row * hidden + c * V);
+  }
+  row_gather<V, THREADS, T>(d1, splits1, split_stride, row, hidden, a);
+  if (d2) row_gather<V, THREADS, T>(d2, splits2, split_stride, row, hidden, b);
+#pragma unroll
+  for (int i = 0; i < kRowSlots; ++i) {
+    const int c = threadIdx.x + i * THREADS;
+    if (c >= nvec) continue;
+#pragma unroll
+    for (int e = 0; e < V; ++e) x[i].v[e] += d2 ? a[i].v[e] + b[i].v[e] : a[i].v[e];
+    row_store<V>(resid + row * hidden + c * V, x[i]);
+    if (cast) row_store<V>(cast + row * hidden + c * V, x[i]);
+  }
+}
+
+// x = resid[row] + delta[row] * rsqrt(mean(delta[row]^2) + deps) * dweight: a product's
+// output that is normed by itself before it joins the stream.  With write_resid the sum
+// is stored back; with `out`, out[r] = x * rsqrt(mean(x^2) + eps) * weight follows in the
+// same pass (the next layer's norm).  rows: as in add_rmsnorm.
+template <typename T, int V, int THREADS>
+__global__ void __launch_bounds__(THREADS)
+    add_normed_rmsnorm_kernel(float* __restrict__ resid, const void* __restrict__ delta, int splits,
+                              const float* __restrict__ dweight, float deps,
+                              const float* __restrict__ weight, float eps, T* __restrict__ out,
+                              const int32_t* __restrict__ rows, int hidden, int write_resid,
+                              size_t split_stride) {
+  __shared__ float scratch[16];
+  const int r = blockIdx.x;
+  const size_t row = rows ? static_cast<size_t>(rows[r]) : static_cast<size_t>(r);
+  const int nvec = hidden / V;
+  RowVec<V> x[kRowSlots], d[kRowSlots];
+#pragma unroll
+  for (int i = 0; i < kRowSlots; ++i) {
+    const int c = threadIdx.x + i * THREADS;
+#pragma unroll
+    for (int e = 0; e < V; ++e) x[i].v[e] = 0.f;
+    if (c < nvec) x[i] = row_load<V>(resid + row * hidden + c * V);
+  }
+  row_gather<V, THREADS, T>(delta, splits, split_stride, row, hidden, d);
+  float ss = 0.f;
+#pragma unroll
+  for (int i = 0; i < kRowSlots; ++i)
+#pragma unroll
+    for (int e = 0; e < V; ++e) ss += d[i].v[e] * d[i].v[e];
+  ss = block_sum(ss, scratch);
+  const float dinv = rsqrtf(ss / static_cast<float>(hidden) + deps);
+  float xx = 0.f;
+#pragma unroll
+  for (int i = 0; i < kRowSlots; ++i) {
+    const int c = threadIdx.x + i * THREADS;
+    if (c >= nvec) continue;
+    const RowVec<V> w = row_load<V>(dweight + c * V);
+#pragma unroll
+    for (int e = 0; e < V; ++e) {
+      x[i].v[e] += (d[i].v[e] * dinv) * w.v[e];
+      xx += x[i].v[e] * x[i].v[e];
+    }
+    if (write_resid) row_store<V>(resid + row * hidden + c * V, x[i]);
+  }
+  if (!out) return;
+  xx = block_sum(xx, scratch);
+  const float inv = rsqrtf(xx / static_cast<float>(hidden) + eps);
+#pragma unroll
+  for (int i = 0; i < kRowSlots; ++i) {
+    const int c = threadIdx.x + i * THREADS;
+    if (c >= nvec) continue;
+    const RowVec<V> w = row_load<V>(weight + c * V);
+    RowVec<V> y;
+#pragma unroll
+    for (int e = 0; e < V; ++e) y.v[e] = (x[i].v[e] * inv) * w.v[e];
+    row_store<V>(out + static_cast<size_t>(r) * hidden + c * V, y);
+  }
+}
+
+// out[r, j] = act(a[r, j]) * table[ids[r], offset + j] for j < width: a gate times a slice
+// of a table row chosen by the token (table rows are ld elements apart).  act as in act_mul.
+template <typename T>
+__global__ void act_mul_rows_kernel(const T* __restrict__ a, const T* __restrict__ table,
+                                    const int32_t* __restrict__ ids, long long ld, int offset,
+                                    T* __restrict__ out, int width, int act) {
+  const size_t row = blockIdx.y;
+  const int j = blockIdx.x * blockDim.x + threadIdx.x;
+  if (j >= width) return;
+  const float g = to_float(a[row * width + j]);
+  const float u = to_float(table[static_cast<long long>(ids[row]) * ld + offset + j]);
+  const float x = act == 2 ? 2.f * 0.7978845608028654f * (g + 0.044715f * g * g * g) : g;
+  const float s = g / (1.f + expf(-x));
+  out[row * width + j] = from_float<T>(s * u);
+}
+
 // dst[i] = src[i], except dst[patch_at + j] = patch[j] for j < patch_n.  Either side
 // may be page-locked host memory: a step's index arrays come to the device, and
 // its chosen tokens go back, without the copy engine, whose hand-overs to and from
@@ -237,7 +412,7 @@ extern "C" int shk_zero_bytes(void* dst, long long bytes, void* stream) {
 }
 
 extern "C" int shk_embed(const void* table, int dtype, const int32_t* ids, float* out, int n,
-                         int hidden, int vocab, void* stream) {
+                         int hidden, int vocab, float scale, void* stream) {
   SHK_REQUIRE(dtype == kF32 || dtype == kBF16, "embed: unknown dtype %d", dtype);
   SHK_REQUIRE(n >= 0 && hidden > 0 && vocab > 0, "embed: bad sizes n=%d hidden=%d vocab=%d", n,
               hidden, vocab);
@@ -246,9 +421,9 @@ extern "C" int shk_embed(const void* table, int dtype, const int32_t* ids, float
   hipStream_t s = static_cast<hipStream_t>(stream);
   const int threads = hidden >= 256 ? 256 : 64;
   if (dtype == kF32)
-    embed_kernel<float><<<n, threads, 0, s>>>(static_cast<const float*>(table), ids, out, hidden);
+    embed_kernel<float><<<n, threads, 0, s>>>(static_cast<const float*>(table), ids, out, hidden, scale);
   else
-    embed_kernel<bf16><<<n, threads, 0, s>>>(static_cast<const bf16*>(table), ids, out, hidden);
+    embed_kernel<bf16><<<n, threads, 0, s>>>(static_cast<const bf16*>(table), ids, out, hidden, scale);
   SHK_LAUNCH_CHECK("embed");
   return 0;
 }
@@ -317,5 +492,100 @@ extern "C" int shk_act_mul(const void* gu, void* out, int dtype, int n, int inte
     act_mul_kernel<bf16><<<grid, 256, 0, s>>>(static_cast<const bf16*>(gu),
                                                static_cast<bf16*>(out), inter, act);
   SHK_LAUNCH_CHECK("act_mul");
+  return 0;
+}
+
+// widths that the register-held row kernels take, and in which form
+static int row_form(int hidden, bool aligned) {
+  if (hidden % 4 == 0 && aligned && hidden <= 256 * 4 * kRowSlots) return 4;
+  if (hidden <= 1024 * kRowSlots) return 1;
+  return 0;
+}
+static bool aligned16(const void* p) { return reinterpret_cast<uintptr_t>(p) % 16 == 0; }
+
+extern "C" int shk_add_rows(float* resid, const float* other, const float* vec, int n, int hidden,
+                            void* stream) {
+  SHK_REQUIRE(n >= 0 && hidden > 0, "add_rows: bad sizes n=%d hidden=%d", n, hidden);
+  if (n == 0 || (!other && !vec)) return 0;
+  SHK_REQUIRE(resid, "add_rows: null pointer");
+  add_rows_kernel<<<n, 256, 0, static_cast<hipStream_t>(stream)>>>(resid, other, vec, hidden);
+  SHK_LAUNCH_CHECK("add_rows");
+  return 0;
+}
+
+extern "C" int shk_add_deltas(float* resid, const void* d1, int splits1, const void* d2, int splits2,
+                              void* cast, int dtype, int n, int hidden, void* stream) {
+  SHK_REQUIRE(dtype == kF32 || dtype == kBF16, "add_deltas: unknown dtype %d", dtype);
+  SHK_REQUIRE(n >= 0 && hidden > 0 && splits1 >= 0 && splits2 >= 0, "add_deltas: bad sizes n=%d hidden=%d",
+              n, hidden);
+  if (n == 0) return 0;
+  SHK_REQUIRE(resid && d1, "add_deltas: null pointer");
+  const int form = row_form(hidden, aligned16(resid) && aligned16(d1) && aligned16(d2) && aligned16(cast));
+  SHK_REQUIRE(form != 0, "add_deltas: rows of %d elements are too wide", hidden);
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  const size_t stride = static_cast<size_t>(n) * hidden;
+#define SHK_GO(T, V, THREADS)                                                                   \
+  add_deltas_kernel<T, V, THREADS><<<n, THREADS, 0, s>>>(resid, d1, splits1, d2, splits2,        \
+                                                         static_cast<T*>(cast), hidden, stride)
+  if (dtype == kF32 && form == 4) SHK_GO(float, 4, 256);
+  else if (dtype == kF32) SHK_GO(float, 1, 1024);
+  else if (form == 4) SHK_GO(bf16, 4, 256);
+  else SHK_GO(bf16, 1, 1024);
+#undef SHK_GO
+  SHK_LAUNCH_CHECK("add_deltas");
+  return 0;
+}
+
+extern "C" int shk_add_normed_rmsnorm(float* resid, const void* delta, int delta_splits,
+                                      const float* dweight, float deps, const float* weight, float eps,
+                                      void* out, int dtype, const int32_t* rows, int n, int hidden,
+                                      int write_resid, int resid_rows, void* stream) {
+  SHK_REQUIRE(dtype == kF32 || dtype == kBF16, "add_normed_rmsnorm: unknown dtype %d", dtype);
+  SHK_REQUIRE(n >= 0 && hidden > 0 && delta_splits >= 0 && resid_rows >= 0,
+              "add_normed_rmsnorm: bad sizes n=%d hidden=%d", n, hidden);
+  SHK_REQUIRE(deps > 0.f && (!out || eps > 0.f), "add_normed_rmsnorm: eps must be > 0");
+  if (n == 0) return 0;
+  SHK_REQUIRE(resid && delta && dweight && (!out || weight), "add_normed_rmsnorm: null pointer");
+  SHK_REQUIRE(out || write_resid, "add_normed_rmsnorm: nothing to write");
+  const int form = row_form(hidden, aligned16(resid) && aligned16(delta) && aligned16(dweight) &&
+                                        aligned16(weight) && aligned16(out));
+  SHK_REQUIRE(form != 0, "add_normed_rmsnorm: rows of %d elements are too wide", hidden);
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  const size_t stride = static_cast<size_t>(resid_rows) * hidden;
+#define SHK_GO(T, V, THREADS)                                                                      \
+  add_normed_rmsnorm_kernel<T, V, THREADS><<<n, THREADS, 0, s>>>(                                   \
+      resid, delta, delta_splits, dweight, deps, weight, eps, static_cast<T*>(out), rows, hidden,   \
+      write_resid, stride)
+  if (dtype == kF32 && form == 4) SHK_GO(float, 4, 256);
+  else if (dtype == kF32) SHK_GO(float, 1, 1024);
+  else if (form == 4) SHK_GO(bf16, 4, 256);
+  else SHK_GO(bf16, 1, 1024);
+#undef SHK_GO
+  SHK_LAUNCH_CHECK("add_normed_rmsnorm");
+  return 0;
+}
+
+extern "C" int shk_act_mul_rows(const void* a, const void* table, int dtype, const int32_t* ids,
+                                long long ld, int offset, int table_rows, void* out, int n, int width,
+                                int act, void* stream) {
+  SHK_REQUIRE(dtype == kF32 || dtype == kBF16, "act_mul_rows: unknown dtype %d", dtype);
+  SHK_REQUIRE(act == 1 || act == 2, "act_mul_rows: unknown activation %d", act);
+  SHK_REQUIRE(n >= 0 && width > 0 && offset >= 0 && ld >= offset + width && table_rows > 0,
+              "act_mul_rows: bad sizes n=%d width=%d offset=%d ld=%lld", n, width, offset, ld);
+  if (n == 0) return 0;
+  SHK_REQUIRE(n <= 65535, "act_mul_rows: at most 65535 rows a call, got %d", n);
+  SHK_REQUIRE(a && table && ids && out, "act_mul_rows: null pointer");
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  const int threads = width >= 256 ? 256 : 64;
+  dim3 grid((width + threads - 1) / threads, n);
+  if (dtype == kF32)
+    act_mul_rows_kernel<float><<<grid, threads, 0, s>>>(static_cast<const float*>(a),
+                                                        static_cast<const float*>(table), ids, ld, offset,
+                                                        static_cast<float*>(out), width, act);
+  else
+    act_mul_rows_kernel<bf16><<<grid, threads, 0, s>>>(static_cast<const bf16*>(a),
+                                                       static_cast<const bf16*>(table), ids, ld, offset,
+                                                       static_cast<bf16*>(out), width, act);
+  SHK_LAUNCH_CHECK("act_mul_rows");
   return 0;
 }

@@ -20,14 +20,16 @@ __global__ void __launch_bounds__(kRopeThreads)
                          int table_stride, T* __restrict__ k_pool, T* __restrict__ v_pool,
                          int page_size, int num_pages, int write_kv,
                          const float* __restrict__ parts, int splits,
-                         const float* __restrict__ bias) {
+                         const float* __restrict__ bias, int adjacent, int v_from_k) {
   __shared__ float cs[kMaxHalf];
   __shared__ float sn[kMaxHalf];
   const int t = blockIdx.x;
   const int pos = positions[t];
   const int half = rot_dim / 2;
-  const int width = (heads + 2 * kv_heads) * head_dim;
+  const int width = (heads + (v_from_k ? 1 : 2) * kv_heads) * head_dim;
   T* row = qkv + static_cast<size_t>(t) * width;
+  // pair i of a head: elements (i, i + half), or the neighbours (2i, 2i + 1)
+  const int partner = adjacent ? 1 : half;
 
   // What this thread moves: a rotated pair, an element behind the rotated part,
   // or an element of the values.  Its inputs are requested first, so that they
@@ -42,7 +44,7 @@ __global__ void __launch_bounds__(kRopeThreads)
   if (item < n_pairs) {
     role = kPairItem;
     h = item / half, i = item % half;
-    col = h * head_dim + i;
+    col = h * head_dim + (adjacent ? 2 * i : i);
   } else if (item < n_pairs + n_tail) {
     role = kTailItem;
     const int e = item - n_pairs;
@@ -51,16 +53,17 @@ __global__ void __launch_bounds__(kRopeThreads)
   } else if (item < n_pairs + n_tail + n_values) {
     role = kValueItem;
     i = item - n_pairs - n_tail;  // kv head * head_dim + element
-    col = (heads + kv_heads) * head_dim + i;
+    // values of their own, or the keys as they were projected (before the rotation)
+    col = (v_from_k ? heads : heads + kv_heads) * head_dim + i;
   }
-  // columns `col` and (for a pair) `col + half` of this token's projections; the
+  // columns `col` and (for a pair) `col + partner` of this token's projections; the
   // parts of a split product are added in order, eight of them in flight
   float x1 = 0.f, x2 = 0.f;
   if (role != kNone) {
     const bool two = role == kPairItem;
     if (splits == 0) {
       x1 = to_float(row[col]);
-      if (two) x2 = to_float(row[col + half]);
+      if (two) x2 = to_float(row[col + partner]);
     } else {
       const size_t split_stride = static_cast<size_t>(n) * width;
       const float* p = parts + static_cast<size_t>(t) * width + col;
@@ -70,7 +73,7 @@ __global__ void __launch_bounds__(kRopeThreads)
         for (int u = 0; u < 8; ++u) {
           const bool have = z0 + u < splits;
           a[u] = have ? p[(z0 + u) * split_stride] : 0.f;
-          b[u] = have && two ? p[(z0 + u) * split_stride + half] : 0.f;
+          b[u] = have && two ? p[(z0 + u) * split_stride + partner] : 0.f;
         }
 #pragma unroll
         for (int u = 0; u < 8; ++u) {
@@ -80,7 +83,7 @@ __global__ void __launch_bounds__(kRopeThreads)
       }
       if (bias) {
         x1 += bias[col];
-        if (two) x2 += bias[col + half];
+        if (two) x2 += bias[col + partner];
       }
     }
   }
@@ -115,11 +118,12 @@ __global__ void __launch_bounds__(kRopeThreads)
     const float o1 = x1 * cs[i] - x2 * sn[i], o2 = x2 * cs[i] + x1 * sn[i];
     if (h < heads) {
       row[col] = from_float<T>(o1);
-      row[col + half] = from_float<T>(o2);
+      row[col + partner] = from_float<T>(o2);
     } else if (page >= 0) {
       T* dst = k_pool + page_base + static_cast<size_t>(h - heads) * page_size * head_dim;
-      dst[key_offset(slot, i, page_size, head_dim)] = from_float<T>(o1);
-      dst[key_offset(slot, i + half, page_size, head_dim)] = from_float<T>(o2);
+      const int e1 = adjacent ? 2 * i : i;
+      dst[key_offset(slot, e1, page_size, head_dim)] = from_float<T>(o1);
+      dst[key_offset(slot, e1 + partner, page_size, head_dim)] = from_float<T>(o2);
     }
   } else if (role == kTailItem) {
     if (h < heads) {
@@ -282,8 +286,9 @@ extern "C" int shk_rope_kv_store(void* qkv, int dtype, int n, int heads, int kv_
                                  const int32_t* tables, int table_stride, void* k_pool,
                                  void* v_pool, int page_size, int num_pages, int write_kv,
                                  const float* parts, int splits, const float* bias,
-                                 void* stream) {
+                                 int pairing, int v_from_k, void* stream) {
   SHK_REQUIRE(dtype == kF32 || dtype == kBF16, "rope_kv_store: unknown dtype %d", dtype);
+  SHK_REQUIRE(pairing == 0 || pairing == 1, "rope_kv_store: unknown pairing %d", pairing);
   SHK_REQUIRE(n >= 0 && heads > 0 && kv_heads > 0 && head_dim > 0,
               "rope_kv_store: bad sizes n=%d heads=%d kv_heads=%d head_dim=%d", n, heads, kv_heads,
               head_dim);
@@ -293,6 +298,7 @@ extern "C" int shk_rope_kv_store(void* qkv, int dtype, int n, int heads, int kv_
               2 * kMaxHalf);
   SHK_REQUIRE(splits >= 0 && (splits == 0 || parts), "rope_kv_store: partial sums without a pointer");
   if (n == 0) return 0;
+  v_from_k = v_from_k != 0;
   SHK_REQUIRE(n <= 2147483647 / ((heads + 2 * kv_heads) * head_dim),
               "rope_kv_store: too many tokens (%d)", n);
   SHK_REQUIRE(qkv && positions, "rope_kv_store: null pointer");
@@ -306,7 +312,8 @@ extern "C" int shk_rope_kv_store(void* qkv, int dtype, int n, int heads, int kv_
   hipStream_t s = static_cast<hipStream_t>(stream);
   // whole vectors where the layout allows: bfloat16, rows rotated whole, 16-byte alignment
   const int vec_items = (heads + kv_heads) * (head_dim / 16) + kv_heads * (head_dim / 8);
-  if (dtype == kBF16 && rot_dim == head_dim && head_dim % 16 == 0 && n >= kVecMinTokens &&
+  if (dtype == kBF16 && pairing == 0 && !v_from_k && rot_dim == head_dim && head_dim % 16 == 0 &&
+      n >= kVecMinTokens &&
       vec_items <= kVecItems * kRopeThreads && reinterpret_cast<uintptr_t>(qkv) % 16 == 0 &&
       (!write_kv || reinterpret_cast<uintptr_t>(k_pool) % 16 == 0) &&
       (!parts || reinterpret_cast<uintptr_t>(parts) % 16 == 0)) {
@@ -324,12 +331,12 @@ extern "C" int shk_rope_kv_store(void* qkv, int dtype, int n, int heads, int kv_
     rope_kv_store_kernel<float><<<grid, kRopeThreads, 0, s>>>(
         static_cast<float*>(qkv), n, heads, kv_heads, head_dim, rot_dim, inv_freq, positions,
         token_seq, tables, table_stride, static_cast<float*>(k_pool), static_cast<float*>(v_pool),
-        page_size, num_pages, write_kv, parts, splits, bias);
+        page_size, num_pages, write_kv, parts, splits, bias, pairing, v_from_k);
   else
     rope_kv_store_kernel<bf16><<<grid, kRopeThreads, 0, s>>>(
         static_cast<bf16*>(qkv), n, heads, kv_heads, head_dim, rot_dim, inv_freq, positions,
         token_seq, tables, table_stride, static_cast<bf16*>(k_pool), static_cast<bf16*>(v_pool),
-        page_size, num_pages, write_kv, parts, splits, bias);
+        page_size, num_pages, write_kv, parts, splits, bias, pairing, v_from_k);
   SHK_LAUNCH_CHECK("rope_kv_store");
   return 0;
 }

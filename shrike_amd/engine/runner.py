@@ -150,8 +150,7 @@ class ModelRunner:
                         f"block table has {len(table)} pages but the step reaches page {last_page}"
                     )
                 # the pages this step writes, and the oldest page it reads
-                w = g.spec.window
-                first = 0 if w is None else max(0, e.start - w + 1) // ps
+                first = g.spec.first_needed(e.start) // ps
                 touched = table[e.start // ps : last_page + 1]
                 if min(touched) < 0 or max(touched) >= self.cache.num_pages or table[first] < 0:
                     raise StepError("block table names a page outside the pool")

@@ -28,7 +28,11 @@ _SIGNATURES = {
     "shk_copy_words": [_P, _P, _I, _P, _I, _I, _P],
     "shk_gather_rows": [_P, c_longlong, _I, _P, _P, _I, _I, _P],
     "shk_zero_bytes": [_P, c_longlong, _P],
-    "shk_embed": [_P, _I, _P, _P, _I, _I, _I, _P],
+    "shk_embed": [_P, _I, _P, _P, _I, _I, _I, _F, _P],
+    "shk_add_rows": [_P, _P, _P, _I, _I, _P],
+    "shk_add_deltas": [_P, _P, _I, _P, _I, _P, _I, _I, _I, _P],
+    "shk_add_normed_rmsnorm": [_P, _P, _I, _P, _F, _P, _F, _P, _I, _P, _I, _I, _I, _I, _P],
+    "shk_act_mul_rows": [_P, _P, _I, _P, c_longlong, _I, _I, _P, _I, _I, _I, _P],
     "shk_add_rmsnorm": [_P, _P, _P, _F, _P, _I, _P, _I, _I, _I, _I, _I, _P],
     "shk_act_mul": [_P, _P, _I, _I, _I, _I, _P],
     "shk_gemm": [_P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _I, _P],
@@ -38,14 +42,15 @@ _SIGNATURES = {
     "shk_gemm_bf16_splits": [_I, _I, _I],
     "shk_gemm_bf16_parts": [_I, _I, _I, _I],
     "shk_mfma_alone": [_P, _P, _I, _I, _P],
-    "shk_rope_kv_store": [_P, _I, _I, _I, _I, _I, _I, _P, _P, _P, _P, _I, _P, _P, _I, _I, _I, _P, _I, _P, _P],
-    "shk_attention": [_P, _I, _P, _I, _I, _I, _I, _I, _P, _P, _P, _I, _I, _P, _P, _I, _I, _I, _F, _P],
+    "shk_rope_kv_store": [_P, _I, _I, _I, _I, _I, _I, _P, _P, _P, _P, _I, _P, _P, _I, _I, _I, _P, _I, _P, _I, _I,
+                          _P],
+    "shk_attention": [_P, _I, _P, _I, _I, _I, _I, _I, _P, _P, _P, _I, _I, _P, _P, _I, _I, _I, _I, _F, _P],
     "shk_attention_supports_mfma": [_I, _I, _I, _I, _I],
-    "shk_attention_decode_bf16": [_P, _I, _P, _I, _I, _I, _I, _P, _P, _I, _P, _P, _I, _I, _F, _P, _I, _I, _P],
-    "shk_attention_prefill_bf16": [_P, _I, _P, _I, _I, _I, _I, _P, _P, _P, _P, _P, _I, _P, _P, _I, _I, _F, _P],
+    "shk_attention_decode_bf16": [_P, _I, _P, _I, _I, _I, _I, _P, _P, _I, _P, _P, _I, _I, _I, _F, _P, _I, _I, _P],
+    "shk_attention_prefill_bf16": [_P, _I, _P, _I, _I, _I, _I, _P, _P, _P, _P, _P, _I, _P, _P, _I, _I, _I, _F, _P],
     "shk_attention_prefill_shared_tiles": [_I, _I, _I, _I],
-    "shk_attention_prefill_shared_bf16": [_P, _I, _P, _I, _I, _I, _I, _P, _P, _P, _P, _P, _I, _P, _P, _I, _I, _F, _I,
-                                          _P, _I, _I, _I, _P],
+    "shk_attention_prefill_shared_bf16": [_P, _I, _P, _I, _I, _I, _I, _P, _P, _P, _P, _P, _I, _P, _P, _I, _I, _I, _F,
+                                          _I, _P, _I, _I, _I, _P],
     "shk_argmax": [_P, _P, _I, _I, _I, _P, _P],
     "shk_argmax_scratch_floats": [_I, _I],
     "shk_sample": [_P, _P, _P, _P, _P, _P, c_longlong, _I, _I, _I, _I, _P],

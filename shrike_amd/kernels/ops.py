@@ -107,17 +107,97 @@ def zero_(t: torch.Tensor) -> None:
     check(load().shk_zero_bytes(_dev(t, "t"), t.numel() * t.element_size(), _stream()))
 
 
-def embed(table: torch.Tensor, ids: torch.Tensor, out: torch.Tensor) -> None:
-    """out[i] = float(table[ids[i]]); ids int32 [n], out float32 [n, hidden]."""
+def embed(table: torch.Tensor, ids: torch.Tensor, out: torch.Tensor, scale: float = 1.0) -> None:
+    """out[i] = float(table[ids[i]]) * scale; ids int32 [n], out float32 [n, hidden]."""
     n, hidden = out.shape
     if not (table.is_contiguous() and out.is_contiguous() and table.shape[1] == hidden):
         raise KernelError("embed: table/out must be contiguous with the same width")
     check(
         load().shk_embed(
             _dev(table, "table"), dtype_code(table.dtype), _dev(ids, "ids", torch.int32),
-            _dev(out, "out", torch.float32), n, hidden, table.shape[0], _stream(),
+            _dev(out, "out", torch.float32), n, hidden, table.shape[0], float(scale), _stream(),
         )
     )
+
+
+def _delta(delta, resid, dtype, who: str):
+    """(address, splits) of a product's output that a row kernel adds to `resid`: a
+    tensor of the compute dtype, or the partial sums of a SplitSum."""
+    if isinstance(delta, SplitSum):
+        if delta.bias is not None or tuple(delta.shape) != tuple(resid.shape):
+            raise KernelError(f"{who}: partial sums must match resid's shape and carry no bias")
+        if delta.parts.dtype != torch.float32 or not delta.parts.is_contiguous():
+            raise KernelError(f"{who}: partial sums must be contiguous float32")
+        return _dev(delta.parts, "delta"), delta.parts.shape[0]
+    if delta.dtype != dtype or not delta.is_contiguous() or delta.shape != resid.shape:
+        raise KernelError(f"{who}: a delta must match resid's shape and have the compute dtype")
+    return _dev(delta, "delta"), 0
+
+
+def add_rows(resid, other=None, vec=None) -> None:
+    """resid[r] += other[r] + vec (float32; either may be None)."""
+    n, hidden = resid.shape
+    if not resid.is_contiguous() or (other is not None and (other.shape != resid.shape or not other.is_contiguous())):
+        raise KernelError("add_rows: resid and other must be contiguous and of one shape")
+    if vec is not None and (vec.numel() != hidden or not vec.is_contiguous()):
+        raise KernelError(f"add_rows: vec has {vec.numel()} elements, hidden is {hidden}")
+    check(load().shk_add_rows(_dev(resid, "resid", torch.float32),
+                              None if other is None else _dev(other, "other", torch.float32),
+                              None if vec is None else _dev(vec, "vec", torch.float32), n, hidden, _stream()))
+
+
+def add_deltas(resid, d1, d2=None, cast=None, dtype=None) -> None:
+    """resid += d1 + d2 (outputs of products: tensors of the compute dtype or SplitSums);
+    cast, if given, receives the new resid in the compute dtype."""
+    n, hidden = resid.shape
+    dtype = cast.dtype if cast is not None else dtype
+    if dtype is None:
+        raise KernelError("add_deltas: give cast or dtype")
+    if not resid.is_contiguous() or (cast is not None and (cast.shape != resid.shape or not cast.is_contiguous())):
+        raise KernelError("add_deltas: resid and cast must be contiguous and of one shape")
+    p1, s1 = _delta(d1, resid, dtype, "add_deltas")
+    p2, s2 = (None, 0) if d2 is None else _delta(d2, resid, dtype, "add_deltas")
+    check(load().shk_add_deltas(_dev(resid, "resid", torch.float32), p1, s1, p2, s2,
+                                None if cast is None else _dev(cast, "cast"), dtype_code(dtype), n, hidden,
+                                _stream()))
+
+
+def add_normed_rmsnorm(resid, delta, dweight, deps: float, weight=None, eps: float = 0.0, out=None,
+                       rows=None, write_resid=True, dtype=None) -> None:
+    """x = resid + delta * rsqrt(mean(delta^2) + deps) * dweight (per row; stored back with
+    write_resid); with `out`, out = x * rsqrt(mean(x^2) + eps) * weight too.  With `rows`
+    (int32 [n]) only those rows, into out[0..n)."""
+    hidden = resid.shape[1]
+    dtype = out.dtype if out is not None else dtype
+    if dtype is None:
+        raise KernelError("add_normed_rmsnorm: give out or dtype")
+    n = resid.shape[0] if rows is None else rows.shape[0]
+    if not resid.is_contiguous() or (out is not None and (tuple(out.shape) != (n, hidden) or not out.is_contiguous())):
+        raise KernelError("add_normed_rmsnorm: resid/out must be contiguous with the same width")
+    if dweight.numel() != hidden or (weight is not None and weight.numel() != hidden):
+        raise KernelError(f"add_normed_rmsnorm: weights must have {hidden} elements")
+    p, splits = _delta(delta, resid, dtype, "add_normed_rmsnorm")
+    check(load().shk_add_normed_rmsnorm(
+        _dev(resid, "resid", torch.float32), p, splits, _dev(dweight, "dweight", torch.float32), float(deps),
+        None if weight is None else _dev(weight, "weight", torch.float32), float(eps),
+        None if out is None else _dev(out, "out"), dtype_code(dtype),
+        None if rows is None else _dev(rows, "rows", torch.int32), n, hidden, int(bool(write_resid)),
+        resid.shape[0], _stream()))
+
+
+def act_mul_rows(a, table, ids, offset: int, out, activation: str) -> None:
+    """out[r, j] = act(a[r, j]) * table[ids[r], offset + j]: a gate times a slice of the
+    table row that the token chooses."""
+    n, width = out.shape
+    if a.shape != out.shape or not a.is_contiguous() or not out.is_contiguous() or a.dtype != out.dtype:
+        raise KernelError("act_mul_rows: a and out must be contiguous, of one shape and dtype")
+    if table.dim() != 2 or not table.is_contiguous() or table.dtype != out.dtype:
+        raise KernelError("act_mul_rows: table must be a contiguous matrix of out's dtype")
+    if offset < 0 or offset + width > table.shape[1] or ids.shape[0] < n:
+        raise KernelError("act_mul_rows: the slice does not fit the table, or too few ids")
+    check(load().shk_act_mul_rows(_dev(a, "a"), _dev(table, "table"), dtype_code(out.dtype),
+                                  _dev(ids, "ids", torch.int32), table.shape[1], int(offset), table.shape[0],
+                                  _dev(out, "out"), n, width, activation_code(activation), _stream()))
 
 
 def add_rmsnorm(resid, delta, weight, eps: float, out, rows=None, write_resid=True) -> None:
@@ -316,13 +396,18 @@ def _check_pools(who, q, tables, k_pool, v_pool, kv_heads, head_dim, page_size) 
 
 
 def rope_kv_store(qkv, heads, kv_heads, head_dim, rot_dim, inv_freq, positions, token_seq,
-                  tables, k_pool, v_pool, page_size, write_kv=True, split_sum=None) -> None:
+                  tables, k_pool, v_pool, page_size, write_kv=True, split_sum=None,
+                  adjacent_pairs: bool = False, values_from_keys: bool = False) -> None:
     """Rotate q and k of qkv [n, (heads + 2 kv_heads) head_dim] in float32 and put
     k, v into their pages (keys in slabs, see key_pool_shape; values transposed
-    [pages, kv_heads, head_dim, page_size])."""
+    [pages, kv_heads, head_dim, page_size]).  adjacent_pairs: element 2i turns with
+    2i + 1 instead of i with i + rot_dim / 2.  values_from_keys: qkv has no value
+    columns, [n, (heads + kv_heads) head_dim], and a token's values are its keys as
+    they come in (before the rotation)."""
     n = qkv.shape[0]
-    if not qkv.is_contiguous() or qkv.shape[1] != (heads + 2 * kv_heads) * head_dim:
-        raise KernelError("rope_kv_store: qkv must be contiguous [n, (heads + 2 kv_heads) head_dim]")
+    if not qkv.is_contiguous() or qkv.shape[1] != (heads + (1 if values_from_keys else 2) * kv_heads) * head_dim:
+        raise KernelError("rope_kv_store: qkv must be contiguous [n, (heads + 2 kv_heads) head_dim] "
+                          "(heads + kv_heads with values_from_keys)")
     # the kernel reads one position (and one sequence index) per row of qkv
     if positions.shape[0] < n or (write_kv and token_seq.shape[0] < n):
         raise KernelError(f"rope_kv_store: qkv has {n} rows but positions / token_seq are shorter")
@@ -348,13 +433,14 @@ def rope_kv_store(qkv, heads, kv_heads, head_dim, rot_dim, inv_freq, positions, 
             _dev(v_pool, "v_pool") if write_kv else None,
             page_size, num_pages, int(bool(write_kv)),
             None if parts is None else _dev(parts, "parts", torch.float32), splits,
-            None if bias is None else _dev(bias, "bias", torch.float32), _stream(),
+            None if bias is None else _dev(bias, "bias", torch.float32),
+            int(bool(adjacent_pairs)), int(bool(values_from_keys)), _stream(),
         )
     )
 
 
 def attention(q, out, heads, kv_heads, head_dim, positions, token_seq, tables, k_pool, v_pool,
-              page_size, window, scale) -> None:
+              page_size, window, scale, chunk=None) -> None:
     """q: [n, >= heads*head_dim] rows (a view into qkv is fine); out [n, heads*head_dim]."""
     _rows(q, "attention q")
     n = q.shape[0]
@@ -367,7 +453,7 @@ def attention(q, out, heads, kv_heads, head_dim, positions, token_seq, tables, k
             head_dim, _dev(positions, "positions", torch.int32),
             _dev(token_seq, "token_seq", torch.int32), _dev(tables, "tables", torch.int32),
             tables.shape[1], tables.shape[0], _dev(k_pool, "k_pool"), _dev(v_pool, "v_pool"),
-            page_size, k_pool.shape[0], int(window or 0), float(scale), _stream(),
+            page_size, k_pool.shape[0], int(window or 0), int(chunk or 0), float(scale), _stream(),
         )
     )
 
@@ -377,7 +463,7 @@ def attention_supports_mfma(heads, kv_heads, head_dim, page_size, q_stride) -> b
 
 
 def attention_decode(q, out, num_seqs, heads, kv_heads, head_dim, positions, tables, k_pool, v_pool,
-                     page_size, window, scale, partial, nsplit, streaming=False) -> None:
+                     page_size, window, scale, partial, nsplit, streaming=False, chunk=None) -> None:
     """bfloat16 MFMA attention for the first num_seqs rows of q, one token per sequence.
     `streaming`: fetch keys and values with non-temporal loads (same result; faster when
     the launch reads tens of megabytes of them)."""
@@ -396,14 +482,14 @@ def attention_decode(q, out, num_seqs, heads, kv_heads, head_dim, positions, tab
             _dev(q, "q"), q.stride(0), _dev(out, "out"), num_seqs, heads, kv_heads, head_dim,
             _dev(positions, "positions", torch.int32), _dev(tables, "tables", torch.int32),
             tables.shape[1], _dev(k_pool, "k_pool"), _dev(v_pool, "v_pool"), page_size,
-            int(window or 0), float(scale), _dev(partial, "partial", torch.float32), nsplit,
+            int(window or 0), int(chunk or 0), float(scale), _dev(partial, "partial", torch.float32), nsplit,
             int(bool(streaming)), _stream(),
         )
     )
 
 
 def attention_prefill(q, out, num_tiles, heads, kv_heads, head_dim, cu_q, ctx_lens, tile_seq, tile_q0,
-                      tables, k_pool, v_pool, page_size, window, scale) -> None:
+                      tables, k_pool, v_pool, page_size, window, scale, chunk=None) -> None:
     """bfloat16 MFMA attention for prompt portions, in tiles of 16 queries."""
     _rows(q, "attention_prefill q")
     if q.dtype != torch.bfloat16 or out.dtype != torch.bfloat16:
@@ -419,7 +505,7 @@ def attention_prefill(q, out, num_tiles, heads, kv_heads, head_dim, cu_q, ctx_le
             _dev(cu_q, "cu_q", torch.int32), _dev(ctx_lens, "ctx_lens", torch.int32),
             _dev(tile_seq, "tile_seq", torch.int32), _dev(tile_q0, "tile_q0", torch.int32),
             _dev(tables, "tables", torch.int32), tables.shape[1], _dev(k_pool, "k_pool"),
-            _dev(v_pool, "v_pool"), page_size, int(window or 0), float(scale), _stream(),
+            _dev(v_pool, "v_pool"), page_size, int(window or 0), int(chunk or 0), float(scale), _stream(),
         )
     )
 
@@ -432,7 +518,7 @@ def attention_prefill_shared_tiles(heads, kv_heads, head_dim, small=False) -> in
 
 def attention_prefill_shared(q, out, num_wgs, heads, kv_heads, head_dim, cu_q, ctx_lens, wg_seq, wg_q0,
                              tables, k_pool, v_pool, page_size, window, scale, small=False,
-                             partial=None, nsplit: int = 1, first_token: int = 0) -> None:
+                             partial=None, nsplit: int = 1, first_token: int = 0, chunk=None) -> None:
     """bfloat16 MFMA attention for prompt portions; one workgroup per (run of query
     tiles, key/value head) shares each chunk of keys among its query heads.
     wg_seq / wg_q0 are in steps of 16 * attention_prefill_shared_tiles(..., small),
@@ -459,7 +545,7 @@ def attention_prefill_shared(q, out, num_wgs, heads, kv_heads, head_dim, cu_q, c
             _dev(cu_q, "cu_q", torch.int32), _dev(ctx_lens, "ctx_lens", torch.int32),
             _dev(wg_seq, "wg_seq", torch.int32), _dev(wg_q0, "wg_q0", torch.int32),
             _dev(tables, "tables", torch.int32), tables.shape[1], _dev(k_pool, "k_pool"),
-            _dev(v_pool, "v_pool"), page_size, int(window or 0), float(scale), int(small),
+            _dev(v_pool, "v_pool"), page_size, int(window or 0), int(chunk or 0), float(scale), int(small),
             _dev(partial, "partial", torch.float32) if nsplit > 1 else None, int(nsplit), int(first_token),
             int(prompt_tokens), _stream(),
         )

@@ -1,4 +1,4 @@
-from . import qwen2  # noqa: F401  (registers Qwen2ForCausalLM)
+from . import mofarax, qwen2  # noqa: F401  (register Mofarax and Qwen2ForCausalLM)
 from .decoder import DecoderModel
 
-__all__ = ["DecoderModel", "qwen2"]
+__all__ = ["DecoderModel", "mofarax", "qwen2"]

@@ -23,6 +23,9 @@ class DecoderModel:
         self.head = build_part("head", spec.head, h, spec.head_name)
         if spec.tie_word_embeddings:
             self.head.tie(self.embedding)
+        # some run adds the embedding's output to the stream again: it is kept
+        self._keep_embedding = any(e.add_embedding for e in spec.schedule)
+        self.stream_vectors: dict = {}
         # the parts whose prepare() does something, in the order they run
         self._preparers = [p for p in self.parts() if type(p).prepare is not Part.prepare]
 
@@ -40,6 +43,8 @@ class DecoderModel:
         out = list(self.embedding.params())
         for block in self.blocks:
             out += block.params()
+        out += [ParamSpec(name, (rows, self.spec.hidden_size), init="vector", keep_float32=True)
+                for name, rows in self.spec.stream_vectors]
         return out + self.final_norm.params() + self.head.params()
 
     def graph_safe(self) -> bool:
@@ -76,6 +81,7 @@ class DecoderModel:
         for block in self.blocks:
             block.check(runtime)
             block.load(tensors, runtime)
+        self.stream_vectors = {name: tensors[name] for name, _rows in self.spec.stream_vectors}
         self.final_norm.load(tensors, runtime)
         self.head.check(runtime)
         self.head.load(tensors, runtime)
@@ -92,7 +98,16 @@ class DecoderModel:
         """Logits float32 [R, vocab] at ctx.out_rows.  `caches[i]` is the
         LayerCache of schedule position i."""
         hidden = HiddenState(self.embedding.forward(ctx))
+        embedded = self.embedding.forward(ctx, into="embedded") if self._keep_embedding else None
         for pos, entry in enumerate(self.spec.schedule):
+            if entry.add_embedding or entry.add_vector is not None:
+                from ..kernels import ops
+
+                hidden.settle(ctx)
+                vector = None
+                if entry.add_vector is not None:
+                    vector = self.stream_vectors[entry.add_vector[0]][entry.add_vector[1]]
+                ops.add_rows(hidden.resid, embedded if entry.add_embedding else None, vector)
             self.blocks[entry.block].forward(ctx, hidden, caches[pos])
         rows = ctx.out_rows
         if rows.shape[0] == 0:

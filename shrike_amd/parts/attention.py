@@ -8,7 +8,7 @@ import numpy as np
 import torch
 
 from ..kernels import ops
-from .base import PAGE, Mixer, PagedSpec, PageTensor, ParamSpec, build_part, register_mixer
+from .base import PAGE, Mixer, PagedSpec, PageTensor, ParamSpec, PositionEncoding, build_part, register_mixer
 
 QUERY_TILE = 16  # queries per tile of the MFMA kernels for prompt portions
 COMPUTE_UNITS = 256  # of an MI355X; compute_units() asks the device that is there
@@ -30,7 +30,8 @@ def compute_units() -> int:
     return _UNITS
 
 
-def kv_cache_spec(num_kv_heads: int, head_dim: int, window: int | None = None) -> PagedSpec:
+def kv_cache_spec(num_kv_heads: int, head_dim: int, window: int | None = None,
+                  chunk: int | None = None) -> PagedSpec:
     """The cache of grouped-query attention, laid out for this file's kernels: per
     page and key/value head the keys in slabs of 32 elements, [head_dim / 32,
     page_size, 32] (a wavefront's operand load for the matrix instruction then
@@ -43,6 +44,7 @@ def kv_cache_spec(num_kv_heads: int, head_dim: int, window: int | None = None) -
         tensors=(PageTensor("k", (num_kv_heads, head_dim // slab, PAGE, slab)),
                  PageTensor("v", (num_kv_heads, head_dim, PAGE))),
         window=window,
+        chunk=chunk,
     )
 
 
@@ -129,6 +131,9 @@ class PagedAttention(Mixer):
     """q/k/v projections (with or without bias), position encoding of q and k,
     cache write, attention over the sequence's pages, output projection
     (reference: shrike/models/qwen.py:111-125, shrike/engine/model_runner.py:63-151).
+    Beyond the reference's model, by the spec: a window, a block-local mask
+    (`chunk`), and values that are the keys before their rotation
+    (`values_from_keys`: no value projection, the cache still holds both).
 
     The three projections are stacked into one [(H + 2 Hkv) D, h] matrix at
     load time; head j of q is rows j*D..(j+1)*D-1 of the q part, as in the
@@ -150,25 +155,28 @@ class PagedAttention(Mixer):
     def params(self):
         s, h = self.spec, self.width
         q, kv = s.num_heads * s.head_dim, s.num_kv_heads * s.head_dim
-        out = [
-            ParamSpec(f"{self.name}.q_proj.weight", (q, h)),
-            ParamSpec(f"{self.name}.k_proj.weight", (kv, h)),
-            ParamSpec(f"{self.name}.v_proj.weight", (kv, h)),
-            ParamSpec(f"{self.name}.o_proj.weight", (h, q)),
-        ]
+        t = self._tensor
+        out = [ParamSpec(t("q"), (q, h)), ParamSpec(t("k"), (kv, h))]
+        if not s.values_from_keys:
+            out.append(ParamSpec(t("v"), (kv, h)))
+        out.append(ParamSpec(t("o"), (h, q)))
         if s.qkv_bias:
-            out += [
-                ParamSpec(f"{self.name}.q_proj.bias", (q,), init="bias", keep_float32=True),
-                ParamSpec(f"{self.name}.k_proj.bias", (kv,), init="bias", keep_float32=True),
-                ParamSpec(f"{self.name}.v_proj.bias", (kv,), init="bias", keep_float32=True),
-            ]
+            out += [ParamSpec(t(f"{r}_bias"), (q if r == "q" else kv,), init="bias", keep_float32=True)
+                    for r in ("q", "k") + (() if s.values_from_keys else ("v",))]
         if s.out_bias:
-            out.append(ParamSpec(f"{self.name}.o_proj.bias", (h,), init="bias", keep_float32=True))
+            out.append(ParamSpec(t("o_bias"), (h,), init="bias", keep_float32=True))
         return out
+
+    _DEFAULT_NAMES = {"q": "q_proj.weight", "k": "k_proj.weight", "v": "v_proj.weight", "o": "o_proj.weight",
+                      "q_bias": "q_proj.bias", "k_bias": "k_proj.bias", "v_bias": "v_proj.bias",
+                      "o_bias": "o_proj.bias"}
+
+    def _tensor(self, role: str) -> str:
+        return self.tensor_name(role, self._DEFAULT_NAMES[role])
 
     def cache_spec(self):
         s = self.spec
-        return kv_cache_spec(s.num_kv_heads, s.head_dim, s.window)
+        return kv_cache_spec(s.num_kv_heads, s.head_dim, s.window, s.chunk)
 
     def check(self, runtime):
         s = self.spec
@@ -181,21 +189,20 @@ class PagedAttention(Mixer):
             raise ValueError(f"{self.name}: head_dim {s.head_dim} is outside 1..256")
         if s.window is not None and s.window < 1:
             raise ValueError(f"{self.name}: window must be positive, got {s.window}")
+        if s.chunk is not None and s.chunk < 1:
+            raise ValueError(f"{self.name}: chunk must be positive, got {s.chunk}")
+        if s.values_from_keys and self.position is not None and \
+                type(self.position).rotary_table is PositionEncoding.rotary_table:
+            raise ValueError(f"{self.name}: values that are the keys before their position encoding need "
+                             "an encoding that the cache-write kernel applies")
 
     def load(self, tensors, runtime):
-        s, n = self.spec, self.name
-        self.w_qkv = runtime.weight(torch.cat(
-            [tensors[f"{n}.q_proj.weight"], tensors[f"{n}.k_proj.weight"], tensors[f"{n}.v_proj.weight"]],
-            dim=0,
-        ))
-        self.b_qkv = (
-            torch.cat([tensors[f"{n}.q_proj.bias"], tensors[f"{n}.k_proj.bias"], tensors[f"{n}.v_proj.bias"]])
-            .contiguous()
-            if s.qkv_bias
-            else None
-        )
-        self.w_o = runtime.weight(tensors[f"{n}.o_proj.weight"])
-        self.b_o = tensors[f"{n}.o_proj.bias"] if s.out_bias else None
+        s, t = self.spec, self._tensor
+        roles = ("q", "k") if s.values_from_keys else ("q", "k", "v")
+        self.w_qkv = runtime.weight(torch.cat([tensors[t(r)] for r in roles], dim=0))
+        self.b_qkv = torch.cat([tensors[t(f"{r}_bias")] for r in roles]).contiguous() if s.qkv_bias else None
+        self.w_o = runtime.weight(tensors[t("o")])
+        self.b_o = tensors[t("o_bias")] if s.out_bias else None
         if self.position is not None:
             self.position.load(tensors, runtime)
         self.linear = runtime.linear
@@ -207,7 +214,7 @@ class PagedAttention(Mixer):
     @property
     def plan_key(self):
         s = self.spec
-        return ("paged_attention", s.num_heads, s.num_kv_heads, s.head_dim, s.window)
+        return ("paged_attention", s.num_heads, s.num_kv_heads, s.head_dim, s.window, s.chunk)
 
     def prepare(self, shape) -> None:
         """Decides once per step and head geometry how attention is launched:
@@ -220,12 +227,15 @@ class PagedAttention(Mixer):
         h, hkv, d = s.num_heads, s.num_kv_heads, s.head_dim
         plan = shape.notes[key] = AttentionPlan()
         plan.mfma = self.dtype == torch.bfloat16 and ops.attention_supports_mfma(
-            h, hkv, d, shape.page_size, (h + 2 * hkv) * d)
+            h, hkv, d, shape.page_size, self._qkv_width())
+        # the most keys that any query reads, where the mask bounds them
+        reach = min(x for x in (s.window, s.chunk, 1 << 40) if x)
         if not plan.mfma:
             return  # the general kernel takes every token alike
         if shape.num_decode:
-            plan.nsplit = decode_splits(shape.num_decode, hkv, shape.max_decode_ctx)
-            plan.streaming = decode_streams(shape.num_decode, hkv, d, shape.max_decode_ctx, s.window)
+            plan.nsplit = decode_splits(shape.num_decode, hkv, min(shape.max_decode_ctx, reach))
+            plan.streaming = decode_streams(shape.num_decode, hkv, d, shape.max_decode_ctx,
+                                            reach if s.window or s.chunk else None)
             shape.launch_key.append((key, plan.nsplit, plan.streaming))
         portions = shape.q_lens[shape.num_decode:]
         if portions.size == 0:
@@ -247,8 +257,8 @@ class PagedAttention(Mixer):
             seqs, q0 = portion_runs(portions, shape.num_decode, QUERY_TILE * tiles)
             # the keys an entry's last query reads: where its portion starts plus its queries
             keys = shape.starts[seqs] + q0 + QUERY_TILE * tiles
-            if s.window:
-                keys = np.minimum(keys, s.window + QUERY_TILE * tiles)
+            if s.window or s.chunk:
+                keys = np.minimum(keys, reach + QUERY_TILE * tiles)
             order = heavy_first(keys)
             seqs, q0 = seqs[order], q0[order]
             plan.portion_splits = portion_splits(int(seqs.size) * hkv, int(keys.mean()))
@@ -259,7 +269,7 @@ class PagedAttention(Mixer):
         plan.count = int(seqs.size)
         # what the launches of the portions depend on beyond the step's sizes
         shape.launch_key.append((key, plan.kernel, plan.small, plan.portion_splits, plan.first_token, plan.count))
-        tag = f"{h}:{hkv}:{d}:{s.window or 0}"
+        tag = f"{h}:{hkv}:{d}:{s.window or 0}:{s.chunk or 0}"
         plan.seq_name, plan.q0_name = f"attention_seq:{tag}", f"attention_q0:{tag}"
         shape.add(plan.seq_name, seqs)
         shape.add(plan.q0_name, q0)
@@ -275,14 +285,14 @@ class PagedAttention(Mixer):
         q = qkv[:, : h * d]
         if not plan.mfma:
             ops.attention(q, out, h, hkv, d, ctx.positions, ctx.token_seq, tables, cache.pools["k"],
-                          cache.pools["v"], cache.page_size, s.window, s.scale)
+                          cache.pools["v"], cache.page_size, s.window, s.scale, chunk=s.chunk)
             return
         if ctx.num_decode:
             partial = ctx.buffer("attn_partial", (ctx.num_decode * h * plan.nsplit * (d + 2),),
                                  torch.float32)
             ops.attention_decode(q, out, ctx.num_decode, h, hkv, d, ctx.positions, tables,
                                  cache.pools["k"], cache.pools["v"], cache.page_size, s.window, s.scale,
-                                 partial, plan.nsplit, plan.streaming)
+                                 partial, plan.nsplit, plan.streaming, chunk=s.chunk)
         if plan.kernel == "shared":
             partial = None
             if plan.portion_splits > 1:
@@ -293,16 +303,22 @@ class PagedAttention(Mixer):
                                          ctx.extras[plan.seq_name], ctx.extras[plan.q0_name], tables,
                                          cache.pools["k"], cache.pools["v"], cache.page_size, s.window,
                                          s.scale, small=plan.small, partial=partial,
-                                         nsplit=plan.portion_splits, first_token=plan.first_token)
+                                         nsplit=plan.portion_splits, first_token=plan.first_token,
+                                         chunk=s.chunk)
         elif plan.kernel == "tiles":
             ops.attention_prefill(q, out, plan.count, h, hkv, d, ctx.cu_q, ctx.ctx_lens,
                                   ctx.extras[plan.seq_name], ctx.extras[plan.q0_name], tables,
-                                  cache.pools["k"], cache.pools["v"], cache.page_size, s.window, s.scale)
+                                  cache.pools["k"], cache.pools["v"], cache.page_size, s.window, s.scale,
+                                  chunk=s.chunk)
+
+    def _qkv_width(self) -> int:
+        s = self.spec
+        return (s.num_heads + (1 if s.values_from_keys else 2) * s.num_kv_heads) * s.head_dim
 
     def forward(self, ctx, x: torch.Tensor, cache) -> torch.Tensor:
         s = self.spec
         n = x.shape[0]
-        qkv_width = (s.num_heads + 2 * s.num_kv_heads) * s.head_dim
+        qkv_width = self._qkv_width()
         table = self.position.rotary_table() if self.position is not None else None
         fused_position = self.position is None or table is not None
         split_sum = None
@@ -322,6 +338,8 @@ class PagedAttention(Mixer):
             qkv, s.num_heads, s.num_kv_heads, s.head_dim, rot_dim, inv_freq, ctx.positions,
             ctx.token_seq, tables, cache.pools["k"], cache.pools["v"], cache.page_size,
             write_kv=cache.owned, split_sum=split_sum,
+            adjacent_pairs=bool(table is not None and getattr(self.position, "adjacent_pairs", False)),
+            values_from_keys=s.values_from_keys,
         )
         attn = ctx.buffer("attn_out", (n, s.num_heads * s.head_dim), ctx.dtype)
         self.attend(ctx, qkv, attn, tables, cache)

@@ -17,6 +17,8 @@ width; it never sees which model it is in.  It declares the tensors it needs
 * Embedding:         forward(ctx) -> float32 [N, width], the residual stream's
                      first value, from ctx.token_ids (and ctx.positions).
 * Head:              forward(ctx, x) -> float32 [R, vocab] from the normed rows.
+* SideInput:         forward(ctx, hidden, x) ; something else that a layer adds to
+                     the stream from the step's tokens (a per-layer token input).
 
 Any part may implement prepare(shape): it is called once per step, before the
 step's metadata goes to the device, with the host-side StepShape; there a part
@@ -79,12 +81,29 @@ class PageTensor:
 @dataclass(frozen=True)
 class PagedSpec:
     """Cache need of a mixer: something per token, kept in pages, for all earlier
-    tokens (window None) or for the last `window` of them.  The cache manager
-    allocates every listed tensor as [layers, pages + 1, *dims] and hands a
-    layer its slice under the tensor's name; it knows nothing else about them."""
+    tokens (window None) or for the last `window` of them; with `chunk`, only for
+    the tokens of the current block of `chunk` positions (blocks counted from
+    position 0).  The cache manager allocates every listed tensor as [layers,
+    pages + 1, *dims] and hands a layer its slice under the tensor's name; it
+    knows nothing else about them."""
 
     tensors: tuple[PageTensor, ...]
     window: int | None = None
+    chunk: int | None = None
+
+    def first_needed(self, position: int) -> int:
+        """The oldest position that a query at `position` (or any later one) still reads."""
+        lo = 0
+        if self.window is not None:
+            lo = max(lo, position - self.window + 1)
+        if self.chunk is not None:
+            lo = max(lo, position // self.chunk * self.chunk)
+        return lo
+
+    @property
+    def bounded(self) -> bool:
+        """Whether old pages fall out of reach as a sequence grows."""
+        return self.window is not None or self.chunk is not None
 
     def __post_init__(self):
         names = [t.name for t in self.tensors]
@@ -102,14 +121,30 @@ class StateSpec:
 
 class HiddenState:
     """The residual stream of a step: `resid` float32 [N, width], plus a part's
-    output `pending` (compute dtype) that has not been added yet.  The next
-    norm adds it while it reads the row anyway."""
+    output `pending` (compute dtype, or the partial sums of a split product) that
+    has not been added yet.  The next norm adds it while it reads the row anyway.
+    `pending_norm` = (weight float32 [width], eps) says that `pending` joins the
+    stream as pending * rsqrt(mean(pending^2) + eps) * weight, row by row."""
 
-    __slots__ = ("resid", "pending")
+    __slots__ = ("resid", "pending", "pending_norm")
 
-    def __init__(self, resid: torch.Tensor, pending: torch.Tensor | None = None):
+    def __init__(self, resid: torch.Tensor, pending: torch.Tensor | None = None, pending_norm=None):
         self.resid = resid
         self.pending = pending
+        self.pending_norm = pending_norm
+
+    def settle(self, ctx) -> None:
+        """Adds what is pending to `resid` now (for a reader that is no norm)."""
+        from ..kernels import ops
+
+        if self.pending is None:
+            return
+        if self.pending_norm is not None:
+            weight, eps = self.pending_norm
+            ops.add_normed_rmsnorm(self.resid, self.pending, weight, eps, dtype=ctx.dtype)
+        else:
+            ops.add_deltas(self.resid, self.pending, dtype=ctx.dtype)
+        self.pending = self.pending_norm = None
 
 
 class Part:
@@ -131,6 +166,13 @@ class Part:
         self.spec = spec
         self.width = width
         self.name = name
+
+    def tensor_name(self, role: str, default: str | None = None) -> str:
+        """Full name of the tensor that plays `role` for this part: the part's name plus
+        the sub-name that the spec's `names` gives the role, else plus `default`
+        (the role itself when none is given); an empty sub-name is the part's own name."""
+        sub = dict(getattr(self.spec, "names", ()) or ()).get(role, role if default is None else default)
+        return f"{self.name}.{sub}" if sub else self.name
 
     def params(self) -> list[ParamSpec]:
         return []
@@ -190,6 +232,15 @@ class Block(Part):
         raise NotImplementedError
 
 
+class SideInput(Part):
+    """Adds to the stream from the step's tokens, after a block's sublayers.  `x` is
+    the stream in the compute dtype as it stands (nothing pending); the part leaves
+    its contribution in hidden.pending (and hidden.pending_norm)."""
+
+    def forward(self, ctx, hidden: HiddenState, x: torch.Tensor) -> None:
+        raise NotImplementedError
+
+
 class Embedding(Part):
     """Built from a spec with `vocab_size`; `table` is what a tied head may share."""
 
@@ -218,6 +269,7 @@ _REGISTRIES: dict[str, dict[str, Callable]] = {
     "block": {},
     "embedding": {},
     "head": {},
+    "side": {},
 }
 
 
@@ -251,6 +303,10 @@ def register_embedding(kind: str, cls) -> None:
 
 def register_head(kind: str, cls) -> None:
     _register("head", kind, cls)
+
+
+def register_side(kind: str, cls) -> None:
+    _register("side", kind, cls)
 
 
 def build_part(family: str, spec, width: int, name: str):

@@ -44,3 +44,55 @@ class PreNormResidualBlock(Block):
 
 
 register_block("prenorm_residual", PreNormResidualBlock)
+
+
+class ParallelResidualBlock(Block):
+    """h = norm(x); x += mixer(h) + ffn(h); then the layer's side input, if it has
+    one, adds to x from the step's tokens.  One norm feeds both sublayers.  The two
+    outputs (tensors, or partial sums of split products) are added to the float32
+    stream by one kernel, which also leaves the stream in the compute dtype for the
+    side input's first product."""
+
+    def __init__(self, spec, width, name):
+        super().__init__(spec, width, name)
+        self.norm = build_part("norm", spec.norm, width, f"{name}.{spec.norm_name}")
+        self.mixer = build_part("mixer", spec.mixer, width, f"{name}.{spec.mixer_name}")
+        self.ffn = build_part("ffn", spec.ffn, width, f"{name}.{spec.ffn_name}") if spec.ffn is not None else None
+        self.side = build_part("side", spec.side, width, f"{name}.{spec.side_name}") if spec.side is not None else None
+        self.parts = tuple(p for p in (self.norm, self.mixer, self.ffn, self.side) if p is not None)
+
+    def params(self):
+        return [p for part in self.parts for p in part.params()]
+
+    def check(self, runtime):
+        for part in self.parts:
+            part.check(runtime)
+
+    @property
+    def graph_safe(self):
+        return all(part.graph_safe for part in self.parts)
+
+    @property
+    def launches_follow_shape(self):
+        return all(part.launches_follow_shape for part in self.parts)
+
+    def load(self, tensors, runtime):
+        for part in self.parts:
+            part.load(tensors, runtime)
+
+    def forward(self, ctx, hidden: HiddenState, cache) -> None:
+        from ..kernels import ops
+
+        h = self.norm.forward(ctx, hidden)
+        mixed = self.mixer.forward(ctx, h, cache)
+        fed = self.ffn.forward(ctx, h) if self.ffn is not None else None
+        if self.side is None and fed is None:
+            hidden.pending = mixed  # the next norm adds it
+            return
+        x = ctx.buffer("stream_cast", hidden.resid.shape, ctx.dtype) if self.side is not None else None
+        ops.add_deltas(hidden.resid, mixed, fed, cast=x, dtype=ctx.dtype)
+        if self.side is not None:
+            self.side.forward(ctx, hidden, x)
+
+
+register_block("parallel_residual", ParallelResidualBlock)

@@ -24,14 +24,14 @@ class LinearHead(Head):
 
     def params(self):
         # With tied weights a file may still carry the output matrix; without, it must.
-        return [ParamSpec(f"{self.name}.weight", (self.spec.vocab_size, self.width),
+        return [ParamSpec(self.tensor_name("weight"), (self.spec.vocab_size, self.width),
                           optional=self.tied_to is not None)]
 
     def load(self, tensors, runtime):
-        w = tensors.get(f"{self.name}.weight")
+        w = tensors.get(self.tensor_name("weight"))
         if w is None:
             if self.tied_to is None or self.tied_to.table is None:
-                raise KeyError(f"{self.name}.weight is absent and the model does not tie its weights")
+                raise KeyError(f"{self.tensor_name('weight')} is absent and the model does not tie its weights")
             w = self.tied_to.table
         self.weight = runtime.weight(w)
         self.linear = runtime.linear

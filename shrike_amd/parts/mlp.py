@@ -18,9 +18,9 @@ class SwiGLU(FeedForward):
     def params(self):
         inter, h = self.spec.intermediate_size, self.width
         return [
-            ParamSpec(f"{self.name}.gate_proj.weight", (inter, h)),
-            ParamSpec(f"{self.name}.up_proj.weight", (inter, h)),
-            ParamSpec(f"{self.name}.down_proj.weight", (h, inter)),
+            ParamSpec(self.tensor_name("gate", "gate_proj.weight"), (inter, h)),
+            ParamSpec(self.tensor_name("up", "up_proj.weight"), (inter, h)),
+            ParamSpec(self.tensor_name("down", "down_proj.weight"), (h, inter)),
         ]
 
     def check(self, runtime):
@@ -32,9 +32,9 @@ class SwiGLU(FeedForward):
         self.inter = int(self.spec.intermediate_size)
         self.activation = self.spec.activation
         self.w_gate_up = runtime.gated_weight(
-            tensors[f"{self.name}.gate_proj.weight"], tensors[f"{self.name}.up_proj.weight"]
+            tensors[self.tensor_name("gate", "gate_proj.weight")], tensors[self.tensor_name("up", "up_proj.weight")]
         )
-        self.w_down = runtime.weight(tensors[f"{self.name}.down_proj.weight"])
+        self.w_down = runtime.weight(tensors[self.tensor_name("down", "down_proj.weight")])
         self.linear_deferred = runtime.linear_deferred
         self.gated_linear = runtime.gated_linear
 

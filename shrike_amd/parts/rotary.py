@@ -14,6 +14,7 @@ class RotaryHalf(PositionEncoding):
     cache-write kernel."""
 
     launches_follow_shape = True
+    adjacent_pairs = False  # pairs are (i, i + rot_dim / 2)
 
     def load(self, tensors, runtime):
         d = int(self.spec.rotary_dim)
@@ -26,3 +27,25 @@ class RotaryHalf(PositionEncoding):
 
 
 register_position("rotary_half", RotaryHalf)
+
+
+class RotaryAdjacent(PositionEncoding):
+    """The same rotation on neighbouring elements: pair i of a head is (2i, 2i + 1),
+    i < rot_dim / 2, and turns by position * theta ** (-2i / rot_dim); elements
+    from rot_dim on pass unchanged.  The rates are formed in float64 and rounded
+    once; the cache-write kernel forms the angle as a float32 product."""
+
+    launches_follow_shape = True
+    adjacent_pairs = True
+
+    def load(self, tensors, runtime):
+        d = int(self.spec.rotary_dim)
+        inv_freq = float(self.spec.theta) ** (-torch.arange(0, d, 2, dtype=torch.float64) / d)
+        self.inv_freq = inv_freq.to(torch.float32).to(runtime.device)
+        self.rot_dim = d
+
+    def rotary_table(self):
+        return self.inv_freq, self.rot_dim
+
+
+register_position("rotary_adjacent", RotaryAdjacent)

@@ -2,7 +2,8 @@
 written out as a model folder (config.json, model.safetensors) that the
 ordinary loader reads back.
 
-Matrices and biases are N(0, 0.02), norm weights 1 + N(0, 0.1).  Every tensor
+Matrices and biases are N(0, 0.02), norm weights 1 + N(0, 0.1) ("norm_zero", a
+norm weight stored around zero: N(0, 0.1)).  Every tensor
 has a generator of its own, seeded from the seed and the tensor's name, so a
 tensor's values do not depend on which other tensors exist.
 """
@@ -19,7 +20,7 @@ from safetensors.torch import save_file
 
 from ..parts.base import ParamSpec
 
-_STD = {"matrix": 0.02, "embedding": 0.02, "bias": 0.02, "norm": 0.1}
+_STD = {"matrix": 0.02, "embedding": 0.02, "bias": 0.02, "norm": 0.1, "norm_zero": 0.1, "vector": 0.02}
 
 #: "reference": the distributions above.  "unit": matrices N(0, 1/fan_in) (the
 #: embedding table N(0, 1)), biases N(0, 0.1): every part's output is as large
@@ -45,7 +46,7 @@ def random_tensor(p: ParamSpec, seed: int, dtype: torch.dtype, device="cpu",
             std = float(p.shape[-1]) ** -0.5
         elif p.init == "embedding":
             std = 1.0
-        elif p.init == "bias":
+        elif p.init in ("bias", "vector"):
             std = 0.1
     elif mode != "reference":
         raise ValueError(f"init mode must be one of {INIT_MODES}, got {mode!r}")
