@@ -56,6 +56,8 @@ BF16_PEAK_FLOPS = 2.5e15
 def matmul_params(cfg) -> tuple[int, int]:
     """(elements of all per-layer matrices, elements of the output matrix)."""
     h, d = cfg.hidden_size, cfg.head_dim
+    if getattr(cfg, "layer_elements", None) is not None:  # a design with other matrices per layer
+        return cfg.layer_elements * cfg.num_hidden_layers, cfg.vocab_size * h
     per_layer = (
         (cfg.num_attention_heads + 2 * cfg.num_key_value_heads) * d * h
         + cfg.num_attention_heads * d * h
@@ -307,15 +309,17 @@ def measure_peaks(device="cuda:0") -> dict:
     return out
 
 
-def kernel_breakdown(engine, steps: int = 3) -> dict:
-    """Microseconds per decode step by kernel: the running requests' next steps
-    run kernel by kernel (no graph) with an event before and after every launch."""
+def kernel_breakdown(engine, steps: int = 3, before_step=None) -> dict:
+    """Microseconds per step by kernel: the running requests' next steps run kernel by
+    kernel (no graph) with an event before and after every launch.  `before_step()` is
+    called ahead of every step (to add the prompt that the step is to take in)."""
     import torch
 
     from shrike_amd.kernels import ops
 
     names = ["embed", "add_rmsnorm", "act_mul", "gemm", "gemm_tiled_weight", "rope_kv_store", "attention",
-             "attention_decode", "attention_prefill", "attention_prefill_shared", "argmax", "sample"]
+             "attention_decode", "attention_prefill", "attention_prefill_shared", "argmax", "sample",
+             "add_deltas", "add_normed_rmsnorm", "act_mul_rows", "add_rows"]
     spans: list[tuple[str, object, object]] = []
     saved = {n: getattr(ops, n) for n in names}
 
@@ -342,9 +346,13 @@ def kernel_breakdown(engine, steps: int = 3) -> dict:
     try:
         for n, fn in saved.items():
             setattr(ops, n, wrap(n, fn))
+        if before_step is not None:
+            before_step()
         engine.step()  # buffers of the kernel-by-kernel path
         spans.clear()
         for _ in range(steps):
+            if before_step is not None:
+                before_step()
             # the device is held back while the host queues the step's launches and
             # events, so that an event pair brackets its kernel and not the host's pace
             torch.cuda.synchronize()
@@ -362,6 +370,76 @@ def kernel_breakdown(engine, steps: int = 3) -> dict:
     for label, a, b in spans:
         total[label] = total.get(label, 0.0) + a.elapsed_time(b) * 1e3 / steps
     return {k: round(v, 1) for k, v in sorted(total.items(), key=lambda kv: -kv[1])}
+
+
+def mofarax_like(qcfg, mask_size: int, side_dim: int):
+    """A Mofarax configuration with the layer sizes of a Qwen2 one (same width, heads,
+    head size, feed-forward width, vocabulary and number of layers; heads rotated whole;
+    the loop runs all layers once, so that the two models run layer for layer), and an
+    object that names its sizes as the formulas of this program expect them."""
+    from types import SimpleNamespace
+
+    from shrike_amd.models.mofarax import MofaraxAttention, MofaraxConfig, MofaraxLayer
+
+    mixer = MofaraxAttention(heads=qcfg.num_attention_heads, kv_heads=qcfg.num_key_value_heads, dim=qcfg.head_dim,
+                             vdim=qcfg.head_dim, scale=qcfg.head_dim**-0.5, mask_size=mask_size,
+                             rot_base=qcfg.rope_theta, rot_dims=qcfg.head_dim)
+    layers = tuple(MofaraxLayer(mixer, qcfg.intermediate_size) for _ in range(qcfg.num_hidden_layers))
+    mcfg = MofaraxConfig(vocab=qcfg.vocab_size, width=qcfg.hidden_size, embedding_scale=8.0,
+                         norm_eps=qcfg.rms_norm_eps, layers=layers, side_dim=side_dim,
+                         loop=(0, qcfg.num_hidden_layers, 1))
+    h, d = qcfg.hidden_size, qcfg.head_dim
+    sizes = SimpleNamespace(
+        hidden_size=h, head_dim=d, num_attention_heads=qcfg.num_attention_heads,
+        num_key_value_heads=qcfg.num_key_value_heads, intermediate_size=qcfg.intermediate_size,
+        num_hidden_layers=qcfg.num_hidden_layers, vocab_size=qcfg.vocab_size,
+        # no value projection; the side input's two matrices
+        layer_elements=(2 * qcfg.num_attention_heads + qcfg.num_key_value_heads) * d * h
+        + 3 * h * qcfg.intermediate_size + 2 * side_dim * h)
+    return mcfg, sizes
+
+
+def run_designs(args, qcfg) -> dict:
+    """Mofarax beside Qwen2 at equal layer sizes, random weights: a prompt of 2,048 tokens
+    in one step, decode steps at batch 1, 8 and 64 from that context, and what each
+    kernel takes in a decode step at batch 8 and in the prompt's step."""
+    import gc
+
+    import torch
+
+    from shrike_amd import SamplingParams
+    from shrike_amd.models import mofarax, qwen2
+
+    mcfg, msizes = mofarax_like(qcfg, args.mask_size, args.side_dim)
+    out = {}
+    for name, spec, sizes in (("qwen2", qwen2.build_spec(qcfg), qcfg), ("mofarax", mofarax.build_spec(mcfg), msizes)):
+        engine = make_engine(sizes, spec, 64, args.seed)
+        rng = random.Random(args.seed + 5)
+
+        def add_prompt(engine=engine, rng=rng, sizes=sizes):
+            engine.add_request([rng.randrange(sizes.vocab_size) for _ in range(PROMPT_LEN)],
+                               SamplingParams(max_new_tokens=1, ignore_eos=True))
+
+        res = {"prefill": run_prefill(engine, sizes, args.seed)}
+        res["prefill_kernels_us"] = kernel_breakdown(engine, steps=2, before_step=add_prompt)
+        for batch in (1, 8, 64):
+            d = run_decode(engine, sizes, batch, args.design_steps, args.warmup, args.seed)
+            res[f"decode_b{batch}"] = {"tok_s": round(d["tok_s"], 1), "ms_per_step": round(d["ms_per_step"], 3),
+                                       "roofline_frac": round(d["gb_s"] / HBM_PEAK_GBS, 3)}
+        # the kernels of a decode step at batch 8
+        sampling = SamplingParams(max_new_tokens=64, ignore_eos=True)
+        for _ in range(8):
+            engine.add_request([rng.randrange(sizes.vocab_size) for _ in range(PROMPT_LEN)], sampling)
+        while engine.scheduler.waiting or not all(r.prefill_done for r in engine.scheduler.running):
+            engine.step()
+        res["decode_b8_kernels_us"] = kernel_breakdown(engine, steps=3)
+        for req in list(engine.scheduler.running):
+            engine.abort(req.req_id)
+        out[name] = res
+        del engine
+        gc.collect()
+        torch.cuda.empty_cache()
+    return out
 
 
 def run_mixed(engine, cfg, decodes: int, budget: int, seed: int) -> dict:
@@ -502,6 +580,13 @@ def main() -> int:
     ap.add_argument("--products", action="store_true",
                     help="instead: time a layer's matrix products at 1 to 2,048 tokens with the engine's kernels "
                          "and, as a yardstick, with the vendor library (prints its own JSON line)")
+    ap.add_argument("--mofarax", action="store_true",
+                    help="instead of the default run: the Mofarax design beside Qwen2 at the layer sizes of "
+                         "--shape, random weights: prompt, decode at batch 1 / 8 / 64, per-kernel times")
+    ap.add_argument("--mask-size", type=int, default=8192, metavar="N",
+                    help="--mofarax: positions per block of its attention (8192: no fewer keys than Qwen2 reads)")
+    ap.add_argument("--side-dim", type=int, default=256, metavar="N", help="--mofarax: width of its per-layer token input")
+    ap.add_argument("--design-steps", type=int, default=300, metavar="K", help="--mofarax: timed decode steps per batch size")
     ap.add_argument("--seed", type=int, default=0)
     args = ap.parse_args()
     if args.gpus != 1:
@@ -530,6 +615,17 @@ def main() -> int:
         raw["num_hidden_layers"] = args.layers
     cfg = Qwen2Config.from_dict(raw)
     spec = build_spec(cfg)
+    if args.mofarax:
+        designs = run_designs(args, cfg)
+        print(json.dumps({
+            "metric": f"Mofarax beside Qwen2 at the Qwen2.5-{args.shape.upper()} layer sizes: prompt tok/s, decode "
+                      "tok/s, us per kernel",
+            "value": designs["mofarax"]["decode_b8"]["tok_s"], "unit": "tok/s", "n_gpus": 1, "higher_is_better": True,
+            "dtype": "bf16", "data": "synthetic: random weights, prompt ids uniform in [0, vocab)",
+            "config": {"shape": args.shape, "layers": cfg.num_hidden_layers, "mask_size": args.mask_size,
+                       "side_dim": args.side_dim, "prompt": PROMPT_LEN, "decode_steps": args.design_steps},
+            "designs": designs}))
+        return 0
     if args.products:
         products = run_products(cfg, [1, 8, 64, 512, PROMPT_LEN])
         print(json.dumps({

@@ -56,8 +56,10 @@ int shk_add_normed_rmsnorm(float* resid, const void* delta, int delta_splits, co
 
 // out[r, j] = act(a[r, j]) * table[ids[r] * ld + offset + j] for j < width: a gate times
 // a slice of the table row that the token chooses.  ids must lie in [0, table_rows).
-int shk_act_mul_rows(const void* a, const void* table, int dtype, const int32_t* ids, long long ld,
-                     int offset, int table_rows, void* out, int n, int width, int act, void* stream);
+// a_splits > 0: a is float32 partial sums [a_splits][n][width], added in order.
+int shk_act_mul_rows(const void* a, int a_splits, const void* table, int dtype, const int32_t* ids,
+                     long long ld, int offset, int table_rows, void* out, int n, int width, int act,
+                     void* stream);
 
 // Residual add fused with RMSNorm.  For each of n rows r (row index rows[r]
 // when `rows` is given, else r):  x = resid[row] (+ delta[row]);  if

@@ -352,7 +352,7 @@ __global__ void __launch_bounds__(kDecodeWaves* kWave)
                             int heads, int kv_heads, const int32_t* __restrict__ positions,
                             const int32_t* __restrict__ tables, int table_stride,
                             const bf16* __restrict__ k_pool, const bf16* __restrict__ v_pool,
-                            int page_size, uint32_t page_magic, int window, int chunk, float scale,
+                            int page_size, uint32_t page_magic, int window, int block, float scale,
                             float* __restrict__ partial, int nsplit) {
   constexpr int NBUF = 2;  // chunk buffers: one computed, one in flight
   constexpr int kStep = 32 * kDecodeWaves;  // keys between two chunks of one wavefront
@@ -365,7 +365,7 @@ __global__ void __launch_bounds__(kDecodeWaves* kWave)
   const PageDiv pd{page_size, page_magic};
   // decode sequences come first in the step: token index == sequence index
   const int pos = positions[seq];
-  const int lo = first_key(pos, window, chunk);
+  const int lo = first_key(pos, window, block);
 
   // this split's keys: chunks of 32 from the chunk that holds `lo`; this
   // wavefront's chunks are those at key_begin, key_begin + kStep, ...
@@ -661,7 +661,7 @@ __global__ void __launch_bounds__(kWave) __attribute__((amdgpu_waves_per_eu(2)))
                              const int32_t* __restrict__ tile_q0,
                              const int32_t* __restrict__ tables, int table_stride,
                              const bf16* __restrict__ k_pool, const bf16* __restrict__ v_pool,
-                             int page_size, int window, int chunk, float scale) {
+                             int page_size, int window, int block, float scale) {
   __shared__ __attribute__((aligned(16))) uint16_t p_lds[16 * kPStride];
   // tiles are listed in token order; the last ones read the most keys, so they start first
   const int tile = gridDim.x - 1 - blockIdx.x, head = blockIdx.y;
@@ -686,10 +686,10 @@ __global__ void __launch_bounds__(kWave) __attribute__((amdgpu_waves_per_eu(2)))
   for (int r = 0; r < 4; ++r) {
     const int qi = kg * 4 + r;
     row_pos[r] = (qi < rows) ? start + q0 + qi : -1;  // rows past the portion read nothing
-    row_lo[r] = first_key(row_pos[r], window, chunk);
+    row_lo[r] = first_key(row_pos[r], window, block);
   }
   const int pos_min = start + q0, pos_max = start + q0 + rows - 1;
-  const int lo_min = first_key(pos_min, window, chunk);
+  const int lo_min = first_key(pos_min, window, block);
 
   float m[4], l[4];
   f32x4 o[D / 16];
@@ -744,7 +744,7 @@ __global__ void __launch_bounds__(WAVES* kWave) __attribute__((amdgpu_waves_per_
                                     const int32_t* __restrict__ wg_q0,
                                     const int32_t* __restrict__ tables, int table_stride,
                                     const bf16* __restrict__ k_pool, const bf16* __restrict__ v_pool,
-                                    int page_size, uint32_t page_magic, int window, int chunk, float scale,
+                                    int page_size, uint32_t page_magic, int window, int block, float scale,
                                     float* __restrict__ partial, int nsplit, int first_token,
                                     int partial_rows) {
   constexpr int U = kUnitsPerWave;
@@ -771,7 +771,7 @@ __global__ void __launch_bounds__(WAVES* kWave) __attribute__((amdgpu_waves_per_
 
   // bounds over the whole workgroup: what has to be staged
   const int pos_min = start + q0, pos_max = start + q_end - 1;
-  const int lo_min = first_key(pos_min, window, chunk);
+  const int lo_min = first_key(pos_min, window, block);
   const int key_begin = lo_min & ~31;
   const int nchunks = (pos_max - key_begin) / 32 + 1;
   // this workgroup's share of the chunks (all of them without splits; none at all
@@ -803,7 +803,7 @@ __global__ void __launch_bounds__(WAVES* kWave) __attribute__((amdgpu_waves_per_
       if (j < unit_rows[u]) qf[u][ds].u = *reinterpret_cast<const uint4*>(qrow + ds * 32);
     }
     q_pos[u] = j < unit_rows[u] ? start + unit_q0[u] + j : -1;
-    q_lo[u] = first_key(q_pos[u], window, chunk);
+    q_lo[u] = first_key(q_pos[u], window, block);
     m[u] = -INFINITY;
     l[u] = 0.f;
 #pragma unroll
@@ -872,13 +872,16 @@ __global__ void __launch_bounds__(WAVES* kWave) __attribute__((amdgpu_waves_per_
   };
 
   // ---- one chunk for this wavefront's units, from LDS buffer `buf`
-  // chunks at or before `last_plain` lie wholly inside what every query of the
-  // workgroup reads (none without a window's lower bound to check)
-  const int last_plain = (window > 0 || chunk > 0) ? -1 : (pos_min + 1 - key_begin) / 32 - 1;
+  // chunks first_plain .. last_plain lie wholly inside what every query of the
+  // workgroup reads: they end at or before its first query and begin at or after the
+  // first key of its last query (a window's or a block's lower bound)
+  const int last_plain = (pos_min + 1 - key_begin) / 32 - 1;
+  const int lo_max = first_key(pos_max, window, block);
+  const int first_plain = lo_max > key_begin ? (lo_max - key_begin + 31) / 32 : 0;
   auto attend = [&](int buf, int chunk) {
     const int kb = key_begin + 32 * chunk;
     const int g0 = kb + g * 8;
-    const bool edge = chunk > last_plain;
+    const bool edge = chunk > last_plain || chunk < first_plain;
     u32x4 kf[2][D / 32];
 #pragma unroll
     for (int t = 0; t < 2; ++t)
@@ -1002,16 +1005,16 @@ template <int D>
 static void launch_decode(dim3 grid, hipStream_t s, const bf16* q, int q_stride, bf16* out,
                           int heads, int kv_heads, const int32_t* positions, const int32_t* tables,
                           int table_stride, const bf16* k_pool, const bf16* v_pool, int page_size,
-                          int window, int chunk, float scale, float* partial, int nsplit, int streaming) {
+                          int window, int block, float scale, float* partial, int nsplit, int streaming) {
   const uint32_t magic = static_cast<uint32_t>(((1ull << 32) + page_size - 1) / page_size);
   if (streaming)
     attention_decode_kernel<D, true><<<grid, kDecodeWaves * kWave, 0, s>>>(
         q, q_stride, out, heads, kv_heads, positions, tables, table_stride, k_pool, v_pool, page_size,
-        magic, window, chunk, scale, partial, nsplit);
+        magic, window, block, scale, partial, nsplit);
   else
     attention_decode_kernel<D, false><<<grid, kDecodeWaves * kWave, 0, s>>>(
         q, q_stride, out, heads, kv_heads, positions, tables, table_stride, k_pool, v_pool, page_size,
-        magic, window, chunk, scale, partial, nsplit);
+        magic, window, block, scale, partial, nsplit);
   if (nsplit > 1)
     attention_merge_kernel<D><<<grid.y * heads, kWave, 0, s>>>(partial, out, nsplit);
 }
@@ -1021,11 +1024,11 @@ static void launch_prefill(dim3 grid, hipStream_t s, const bf16* q, int q_stride
                            int heads, int kv_heads, const int32_t* cu_q, const int32_t* ctx_lens,
                            const int32_t* tile_seq, const int32_t* tile_q0, const int32_t* tables,
                            int table_stride, const bf16* k_pool, const bf16* v_pool, int page_size,
-                           int window, int chunk, float scale) {
+                           int window, int block, float scale) {
   attention_prefill_kernel<D><<<grid, kWave, 0, s>>>(q, q_stride, out, heads, kv_heads, cu_q,
                                                      ctx_lens, tile_seq, tile_q0, tables,
                                                      table_stride, k_pool, v_pool, page_size,
-                                                     window, chunk, scale);
+                                                     window, block, scale);
 }
 
 template <int D>
@@ -1033,7 +1036,7 @@ static void launch_prefill_shared(dim3 grid, hipStream_t s, const bf16* q, int q
                                   int heads, int kv_heads, int tiles, const int32_t* cu_q,
                                   const int32_t* ctx_lens, const int32_t* wg_seq,
                                   const int32_t* wg_q0, const int32_t* tables, int table_stride,
-                                  const bf16* k_pool, const bf16* v_pool, int page_size, int window, int chunk,
+                                  const bf16* k_pool, const bf16* v_pool, int page_size, int window, int block,
                                   float scale, bool small, float* partial, int nsplit,
                                   int first_token, int prompt_tokens) {
   const uint32_t magic = static_cast<uint32_t>(((1ull << 32) + page_size - 1) / page_size);
@@ -1041,12 +1044,12 @@ static void launch_prefill_shared(dim3 grid, hipStream_t s, const bf16* q, int q
   if (small)
     attention_prefill_shared_kernel<D, kSharedWavesSmall><<<grid, kSharedWavesSmall * kWave, 0, s>>>(
         q, q_stride, out, heads, kv_heads, tiles, cu_q, ctx_lens, wg_seq, wg_q0, tables,
-        table_stride, k_pool, v_pool, page_size, magic, window, chunk, scale, partial, nsplit, first_token,
+        table_stride, k_pool, v_pool, page_size, magic, window, block, scale, partial, nsplit, first_token,
         rows);
   else
     attention_prefill_shared_kernel<D, kSharedWaves><<<grid, kSharedWaves * kWave, 0, s>>>(
         q, q_stride, out, heads, kv_heads, tiles, cu_q, ctx_lens, wg_seq, wg_q0, tables,
-        table_stride, k_pool, v_pool, page_size, magic, window, chunk, scale, partial, nsplit, first_token,
+        table_stride, k_pool, v_pool, page_size, magic, window, block, scale, partial, nsplit, first_token,
         rows);
   if (nsplit > 1)
     attention_merge_kernel<D><<<rows, kWave, 0, s>>>(
@@ -1093,7 +1096,7 @@ extern "C" int shk_attention_decode_bf16(const void* q, int q_stride, void* out,
                                          int heads, int kv_heads, int head_dim,
                                          const int32_t* positions, const int32_t* tables,
                                          int table_stride, const void* k_pool, const void* v_pool,
-                                         int page_size, int window, int chunk, float scale, float* partial,
+                                         int page_size, int window, int block, float scale, float* partial,
                                          int nsplit, int streaming, void* stream) {
   if (check_mfma_shapes("attention_decode", heads, kv_heads, head_dim, page_size, q_stride)) return 1;
   SHK_REQUIRE(heads / kv_heads <= 16, "attention_decode: at most 16 query heads per key/value head");
@@ -1114,7 +1117,7 @@ extern "C" int shk_attention_decode_bf16(const void* q, int q_stride, void* out,
 #define CALL(D)                                                                              \
   launch_decode<D>(grid, s, static_cast<const bf16*>(q), q_stride, static_cast<bf16*>(out), heads, \
                    kv_heads, positions, tables, table_stride, static_cast<const bf16*>(k_pool),    \
-                   static_cast<const bf16*>(v_pool), page_size, window, chunk, scale, partial, nsplit,    \
+                   static_cast<const bf16*>(v_pool), page_size, window, block, scale, partial, nsplit,    \
                    streaming)
   SHK_DISPATCH_D(head_dim, CALL)
 #undef CALL
@@ -1137,7 +1140,7 @@ extern "C" int shk_attention_prefill_shared_bf16(const void* q, int q_stride, vo
                                                  const int32_t* ctx_lens, const int32_t* wg_seq,
                                                  const int32_t* wg_q0, const int32_t* tables,
                                                  int table_stride, const void* k_pool,
-                                                 const void* v_pool, int page_size, int window, int chunk,
+                                                 const void* v_pool, int page_size, int window, int block,
                                                  float scale, int small, float* partial, int nsplit,
                                                  int first_token, int prompt_tokens, void* stream) {
   if (check_mfma_shapes("attention_prefill_shared", heads, kv_heads, head_dim, page_size, q_stride))
@@ -1169,7 +1172,7 @@ extern "C" int shk_attention_prefill_shared_bf16(const void* q, int q_stride, vo
   launch_prefill_shared<D>(grid, s, static_cast<const bf16*>(q), q_stride, static_cast<bf16*>(out), \
                            heads, kv_heads, tiles, cu_q, ctx_lens, wg_seq, wg_q0, tables,      \
                            table_stride, static_cast<const bf16*>(k_pool),                     \
-                           static_cast<const bf16*>(v_pool), page_size, window, chunk, scale, small != 0, \
+                           static_cast<const bf16*>(v_pool), page_size, window, block, scale, small != 0, \
                            partial, nsplit, first_token, prompt_tokens)
   switch (head_dim) {
     case 32: CALL(32); break;
@@ -1189,7 +1192,7 @@ extern "C" int shk_attention_prefill_bf16(const void* q, int q_stride, void* out
                                           const int32_t* tile_seq, const int32_t* tile_q0,
                                           const int32_t* tables, int table_stride,
                                           const void* k_pool, const void* v_pool, int page_size,
-                                          int window, int chunk, float scale, void* stream) {
+                                          int window, int block, float scale, void* stream) {
   if (check_mfma_shapes("attention_prefill", heads, kv_heads, head_dim, page_size, q_stride)) return 1;
   SHK_REQUIRE(num_tiles >= 0 && heads <= 65535, "attention_prefill: bad sizes");
   if (num_tiles == 0) return 0;
@@ -1203,7 +1206,7 @@ extern "C" int shk_attention_prefill_bf16(const void* q, int q_stride, void* out
   launch_prefill<D>(grid, s, static_cast<const bf16*>(q), q_stride, static_cast<bf16*>(out), \
                     heads, kv_heads, cu_q, ctx_lens, tile_seq, tile_q0, tables, table_stride, \
                     static_cast<const bf16*>(k_pool), static_cast<const bf16*>(v_pool),      \
-                    page_size, window, chunk, scale)
+                    page_size, window, block, scale)
   SHK_DISPATCH_D(head_dim, CALL)
 #undef CALL
   SHK_LAUNCH_CHECK("attention_prefill");

@@ -164,9 +164,8 @@ __global__ void act_mul_kernel(const T* __restrict__ gu, T* __restrict__ out, in
 // ------------------------------------------------- rows held in registers
 // The kernels below keep one row per workgroup in registers: V elements per access
 // (4: whole vectors, for widths that are a multiple of 4 and aligned buffers; 1:
-// every other width), kRowSlots accesses per thread, THREADS threads.
-
-constexpr int kRowSlots = 8;
+// every other width), S accesses per thread, THREADS threads; V * S * THREADS
+// elements fit.  Wide rows get 1024 threads, so that few loads follow each other.
 
 template <int V>
 struct RowVec {
@@ -194,27 +193,46 @@ __device__ __forceinline__ void row_store(T* p, const RowVec<V>& r) {
   }
 }
 
-// The sum of a product's output for one row: a tensor of T (splits 0) or the float32
-// partial sums [splits][rows][hidden] of a product split along k, added in order.
-template <int V, int THREADS, typename T>
+// The output of a product for one row: a tensor of T (splits 0) or the float32
+// partial sums [splits][rows][hidden] of a product split along k, added in order,
+// four parts in flight.
+template <int V, int THREADS, int S, typename T>
 __device__ __forceinline__ void row_gather(const void* delta, int splits, size_t split_stride,
-                                           size_t row, int hidden, RowVec<V> (&d)[kRowSlots]) {
+                                           size_t row, int hidden, RowVec<V> (&d)[S]) {
   const int nvec = hidden / V;
 #pragma unroll
-  for (int i = 0; i < kRowSlots; ++i) {
-    const int c = threadIdx.x + i * THREADS;
+  for (int i = 0; i < S; ++i)
 #pragma unroll
     for (int e = 0; e < V; ++e) d[i].v[e] = 0.f;
-    if (c >= nvec) continue;
-    if (splits == 0) {
-      d[i] = row_load<V>(static_cast<const T*>(delta) + row * hidden + c * V);
-    } else {
-      const float* p = static_cast<const float*>(delta) + row * hidden + c * V;
-      for (int z = 0; z < splits; ++z) {
-        const RowVec<V> more = row_load<V>(p + z * split_stride);
+  if (splits == 0) {
 #pragma unroll
-        for (int e = 0; e < V; ++e) d[i].v[e] += more.v[e];
+    for (int i = 0; i < S; ++i) {
+      const int c = threadIdx.x + i * THREADS;
+      if (c < nvec) d[i] = row_load<V>(static_cast<const T*>(delta) + row * hidden + c * V);
+    }
+    return;
+  }
+  const float* p = static_cast<const float*>(delta) + row * hidden;
+  for (int z0 = 0; z0 < splits; z0 += 4) {
+    RowVec<V> more[4][S];
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      const int z = z0 + u < splits ? z0 + u : splits - 1;  // past the last part: the last again, not added
+#pragma unroll
+      for (int i = 0; i < S; ++i) {
+        const int c = threadIdx.x + i * THREADS;
+#pragma unroll
+        for (int e = 0; e < V; ++e) more[u][i].v[e] = 0.f;
+        if (c < nvec) more[u][i] = row_load<V>(p + z * split_stride + c * V);
       }
+    }
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      const bool have = z0 + u < splits;
+#pragma unroll
+      for (int i = 0; i < S; ++i)
+#pragma unroll
+        for (int e = 0; e < V; ++e) d[i].v[e] += have ? more[u][i].v[e] : 0.f;
     }
   }
 }
@@ -235,27 +253,29 @@ __global__ void __launch_bounds__(256)
 
 // resid[r] += d1[r] + d2[r]; cast[r] = T(resid[r]).  d1 and d2 are outputs of products
 // (see row_gather); d2 and cast may be absent.  (d1 + d2) is formed first, then added.
-template <typename T, int V, int THREADS>
+template <typename T, int V, int THREADS, int S>
 __global__ void __launch_bounds__(THREADS)
     add_deltas_kernel(float* __restrict__ resid, const void* __restrict__ d1, int splits1,
                       const void* __restrict__ d2, int splits2, T* __restrict__ cast, int hidden,
                       size_t split_stride) {
   const size_t row = blockIdx.x;
   const int nvec = hidden / V;
-  RowVec<V> a[kRowSlots], b[kRowSlots], x[kRowSlots];
+  RowVec<V> a[S], b[S], x[S];
 #pragma unroll
-  for (int i = 0; i < kRowSlots; ++i) {
+  for (int i = 0; i < S; ++i) {
     const int c = threadIdx.x + i * THREADS;
+#pragma unroll
+    for (int e = 0; e < V; ++e) x[i].v[e] = b[i].v[e] = 0.f;
     if (c < nvec) x[i] = row_load<V>(resid + row * hidden + c * V);
   }
-  row_gather<V, THREADS, T>(d1, splits1, split_stride, row, hidden, a);
-  if (d2) row_gather<V, THREADS, T>(d2, splits2, split_stride, row, hidden, b);
+  row_gather<V, THREADS, S, T>(d1, splits1, split_stride, row, hidden, a);
+  if (d2) row_gather<V, THREADS, S, T>(d2, splits2, split_stride, row, hidden, b);
 #pragma unroll
-  for (int i = 0; i < kRowSlots; ++i) {
+  for (int i = 0; i < S; ++i) {
     const int c = threadIdx.x + i * THREADS;
     if (c >= nvec) continue;
 #pragma unroll
-    for (int e = 0; e < V; ++e) x[i].v[e] += d2 ? a[i].v[e] + b[i].v[e] : a[i].v[e];
+    for (int e = 0; e < V; ++e) x[i].v[e] += a[i].v[e] + b[i].v[e];
     row_store<V>(resid + row * hidden + c * V, x[i]);
     if (cast) row_store<V>(cast + row * hidden + c * V, x[i]);
   }
@@ -265,7 +285,7 @@ __global__ void __launch_bounds__(THREADS)
 // output that is normed by itself before it joins the stream.  With write_resid the sum
 // is stored back; with `out`, out[r] = x * rsqrt(mean(x^2) + eps) * weight follows in the
 // same pass (the next layer's norm).  rows: as in add_rmsnorm.
-template <typename T, int V, int THREADS>
+template <typename T, int V, int THREADS, int S>
 __global__ void __launch_bounds__(THREADS)
     add_normed_rmsnorm_kernel(float* __restrict__ resid, const void* __restrict__ delta, int splits,
                               const float* __restrict__ dweight, float deps,
@@ -276,31 +296,34 @@ __global__ void __launch_bounds__(THREADS)
   const int r = blockIdx.x;
   const size_t row = rows ? static_cast<size_t>(rows[r]) : static_cast<size_t>(r);
   const int nvec = hidden / V;
-  RowVec<V> x[kRowSlots], d[kRowSlots];
+  RowVec<V> x[S], d[S], dw[S], w[S];
 #pragma unroll
-  for (int i = 0; i < kRowSlots; ++i) {
+  for (int i = 0; i < S; ++i) {
     const int c = threadIdx.x + i * THREADS;
 #pragma unroll
-    for (int e = 0; e < V; ++e) x[i].v[e] = 0.f;
-    if (c < nvec) x[i] = row_load<V>(resid + row * hidden + c * V);
+    for (int e = 0; e < V; ++e) x[i].v[e] = dw[i].v[e] = w[i].v[e] = 0.f;
+    if (c < nvec) {
+      x[i] = row_load<V>(resid + row * hidden + c * V);
+      dw[i] = row_load<V>(dweight + c * V);
+      if (out) w[i] = row_load<V>(weight + c * V);
+    }
   }
-  row_gather<V, THREADS, T>(delta, splits, split_stride, row, hidden, d);
+  row_gather<V, THREADS, S, T>(delta, splits, split_stride, row, hidden, d);
   float ss = 0.f;
 #pragma unroll
-  for (int i = 0; i < kRowSlots; ++i)
+  for (int i = 0; i < S; ++i)
 #pragma unroll
     for (int e = 0; e < V; ++e) ss += d[i].v[e] * d[i].v[e];
   ss = block_sum(ss, scratch);
   const float dinv = rsqrtf(ss / static_cast<float>(hidden) + deps);
   float xx = 0.f;
 #pragma unroll
-  for (int i = 0; i < kRowSlots; ++i) {
+  for (int i = 0; i < S; ++i) {
     const int c = threadIdx.x + i * THREADS;
     if (c >= nvec) continue;
-    const RowVec<V> w = row_load<V>(dweight + c * V);
 #pragma unroll
     for (int e = 0; e < V; ++e) {
-      x[i].v[e] += (d[i].v[e] * dinv) * w.v[e];
+      x[i].v[e] += (d[i].v[e] * dinv) * dw[i].v[e];
       xx += x[i].v[e] * x[i].v[e];
     }
     if (write_resid) row_store<V>(resid + row * hidden + c * V, x[i]);
@@ -309,28 +332,41 @@ __global__ void __launch_bounds__(THREADS)
   xx = block_sum(xx, scratch);
   const float inv = rsqrtf(xx / static_cast<float>(hidden) + eps);
 #pragma unroll
-  for (int i = 0; i < kRowSlots; ++i) {
+  for (int i = 0; i < S; ++i) {
     const int c = threadIdx.x + i * THREADS;
     if (c >= nvec) continue;
-    const RowVec<V> w = row_load<V>(weight + c * V);
     RowVec<V> y;
 #pragma unroll
-    for (int e = 0; e < V; ++e) y.v[e] = (x[i].v[e] * inv) * w.v[e];
+    for (int e = 0; e < V; ++e) y.v[e] = (x[i].v[e] * inv) * w[i].v[e];
     row_store<V>(out + static_cast<size_t>(r) * hidden + c * V, y);
   }
 }
 
 // out[r, j] = act(a[r, j]) * table[ids[r], offset + j] for j < width: a gate times a slice
-// of a table row chosen by the token (table rows are ld elements apart).  act as in act_mul.
+// of a table row chosen by the token (table rows are ld elements apart).  act as in
+// act_mul.  splits > 0: a is the float32 partial sums [splits][n][width] of a product
+// split along k, added in order.
 template <typename T>
-__global__ void act_mul_rows_kernel(const T* __restrict__ a, const T* __restrict__ table,
-                                    const int32_t* __restrict__ ids, long long ld, int offset,
-                                    T* __restrict__ out, int width, int act) {
+__global__ void act_mul_rows_kernel(const void* __restrict__ a, int splits, size_t split_stride,
+                                    const T* __restrict__ table, const int32_t* __restrict__ ids,
+                                    long long ld, int offset, T* __restrict__ out, int width, int act) {
   const size_t row = blockIdx.y;
   const int j = blockIdx.x * blockDim.x + threadIdx.x;
   if (j >= width) return;
-  const float g = to_float(a[row * width + j]);
   const float u = to_float(table[static_cast<long long>(ids[row]) * ld + offset + j]);
+  float g = 0.f;
+  if (splits == 0) {
+    g = to_float(static_cast<const T*>(a)[row * width + j]);
+  } else {
+    const float* p = static_cast<const float*>(a) + row * width + j;
+    for (int z0 = 0; z0 < splits; z0 += 8) {  // eight parts in flight
+      float part[8];
+#pragma unroll
+      for (int q = 0; q < 8; ++q) part[q] = p[(z0 + q < splits ? z0 + q : splits - 1) * split_stride];
+#pragma unroll
+      for (int q = 0; q < 8; ++q) g += z0 + q < splits ? part[q] : 0.f;
+    }
+  }
   const float x = act == 2 ? 2.f * 0.7978845608028654f * (g + 0.044715f * g * g * g) : g;
   const float s = g / (1.f + expf(-x));
   out[row * width + j] = from_float<T>(s * u);
@@ -495,13 +531,27 @@ extern "C" int shk_act_mul(const void* gu, void* out, int dtype, int n, int inte
   return 0;
 }
 
-// widths that the register-held row kernels take, and in which form
+// Which form of the register-held row kernels takes a width: 4 x 256 x 2, 4 x 512 x 2,
+// 4 x 1024 x 2 (whole vectors), 1 x 256 x 4 or 1 x 1024 x 8 elements; 0: too wide.
 static int row_form(int hidden, bool aligned) {
-  if (hidden % 4 == 0 && aligned && hidden <= 256 * 4 * kRowSlots) return 4;
-  if (hidden <= 1024 * kRowSlots) return 1;
+  if (hidden % 4 == 0 && aligned && hidden <= 4 * 256 * 2) return 1;
+  if (hidden % 4 == 0 && aligned && hidden <= 4 * 512 * 2) return 5;
+  if (hidden % 4 == 0 && aligned && hidden <= 4 * 1024 * 2) return 2;
+  if (hidden <= 256 * 4) return 3;
+  if (hidden <= 1024 * 8) return 4;
   return 0;
 }
 static bool aligned16(const void* p) { return reinterpret_cast<uintptr_t>(p) % 16 == 0; }
+
+// SHK_ROW_FORMS(GO, T): GO(T, V, THREADS, S) for the form that row_form chose
+#define SHK_ROW_FORMS(GO, T)        \
+  do {                              \
+    if (form == 1) GO(T, 4, 256, 2);       \
+    else if (form == 5) GO(T, 4, 512, 2);  \
+    else if (form == 2) GO(T, 4, 1024, 2); \
+    else if (form == 3) GO(T, 1, 256, 4);  \
+    else GO(T, 1, 1024, 8);                \
+  } while (0)
 
 extern "C" int shk_add_rows(float* resid, const float* other, const float* vec, int n, int hidden,
                             void* stream) {
@@ -524,13 +574,11 @@ extern "C" int shk_add_deltas(float* resid, const void* d1, int splits1, const v
   SHK_REQUIRE(form != 0, "add_deltas: rows of %d elements are too wide", hidden);
   hipStream_t s = static_cast<hipStream_t>(stream);
   const size_t stride = static_cast<size_t>(n) * hidden;
-#define SHK_GO(T, V, THREADS)                                                                   \
-  add_deltas_kernel<T, V, THREADS><<<n, THREADS, 0, s>>>(resid, d1, splits1, d2, splits2,        \
-                                                         static_cast<T*>(cast), hidden, stride)
-  if (dtype == kF32 && form == 4) SHK_GO(float, 4, 256);
-  else if (dtype == kF32) SHK_GO(float, 1, 1024);
-  else if (form == 4) SHK_GO(bf16, 4, 256);
-  else SHK_GO(bf16, 1, 1024);
+#define SHK_GO(T, V, THREADS, S)                                                                 \
+  add_deltas_kernel<T, V, THREADS, S><<<n, THREADS, 0, s>>>(resid, d1, splits1, d2, splits2,     \
+                                                            static_cast<T*>(cast), hidden, stride)
+  if (dtype == kF32) SHK_ROW_FORMS(SHK_GO, float);
+  else SHK_ROW_FORMS(SHK_GO, bf16);
 #undef SHK_GO
   SHK_LAUNCH_CHECK("add_deltas");
   return 0;
@@ -552,40 +600,37 @@ extern "C" int shk_add_normed_rmsnorm(float* resid, const void* delta, int delta
   SHK_REQUIRE(form != 0, "add_normed_rmsnorm: rows of %d elements are too wide", hidden);
   hipStream_t s = static_cast<hipStream_t>(stream);
   const size_t stride = static_cast<size_t>(resid_rows) * hidden;
-#define SHK_GO(T, V, THREADS)                                                                      \
-  add_normed_rmsnorm_kernel<T, V, THREADS><<<n, THREADS, 0, s>>>(                                   \
-      resid, delta, delta_splits, dweight, deps, weight, eps, static_cast<T*>(out), rows, hidden,   \
+#define SHK_GO(T, V, THREADS, S)                                                                      \
+  add_normed_rmsnorm_kernel<T, V, THREADS, S><<<n, THREADS, 0, s>>>(                                   \
+      resid, delta, delta_splits, dweight, deps, weight, eps, static_cast<T*>(out), rows, hidden,      \
       write_resid, stride)
-  if (dtype == kF32 && form == 4) SHK_GO(float, 4, 256);
-  else if (dtype == kF32) SHK_GO(float, 1, 1024);
-  else if (form == 4) SHK_GO(bf16, 4, 256);
-  else SHK_GO(bf16, 1, 1024);
+  if (dtype == kF32) SHK_ROW_FORMS(SHK_GO, float);
+  else SHK_ROW_FORMS(SHK_GO, bf16);
 #undef SHK_GO
   SHK_LAUNCH_CHECK("add_normed_rmsnorm");
   return 0;
 }
 
-extern "C" int shk_act_mul_rows(const void* a, const void* table, int dtype, const int32_t* ids,
-                                long long ld, int offset, int table_rows, void* out, int n, int width,
-                                int act, void* stream) {
+extern "C" int shk_act_mul_rows(const void* a, int a_splits, const void* table, int dtype,
+                                const int32_t* ids, long long ld, int offset, int table_rows, void* out,
+                                int n, int width, int act, void* stream) {
   SHK_REQUIRE(dtype == kF32 || dtype == kBF16, "act_mul_rows: unknown dtype %d", dtype);
   SHK_REQUIRE(act == 1 || act == 2, "act_mul_rows: unknown activation %d", act);
-  SHK_REQUIRE(n >= 0 && width > 0 && offset >= 0 && ld >= offset + width && table_rows > 0,
+  SHK_REQUIRE(n >= 0 && width > 0 && offset >= 0 && ld >= offset + width && table_rows > 0 && a_splits >= 0,
               "act_mul_rows: bad sizes n=%d width=%d offset=%d ld=%lld", n, width, offset, ld);
   if (n == 0) return 0;
   SHK_REQUIRE(n <= 65535, "act_mul_rows: at most 65535 rows a call, got %d", n);
   SHK_REQUIRE(a && table && ids && out, "act_mul_rows: null pointer");
   hipStream_t s = static_cast<hipStream_t>(stream);
   const int threads = width >= 256 ? 256 : 64;
+  const size_t stride = static_cast<size_t>(n) * width;
   dim3 grid((width + threads - 1) / threads, n);
   if (dtype == kF32)
-    act_mul_rows_kernel<float><<<grid, threads, 0, s>>>(static_cast<const float*>(a),
-                                                        static_cast<const float*>(table), ids, ld, offset,
-                                                        static_cast<float*>(out), width, act);
+    act_mul_rows_kernel<float><<<grid, threads, 0, s>>>(a, a_splits, stride, static_cast<const float*>(table),
+                                                        ids, ld, offset, static_cast<float*>(out), width, act);
   else
-    act_mul_rows_kernel<bf16><<<grid, threads, 0, s>>>(static_cast<const bf16*>(a),
-                                                       static_cast<const bf16*>(table), ids, ld, offset,
-                                                       static_cast<bf16*>(out), width, act);
+    act_mul_rows_kernel<bf16><<<grid, threads, 0, s>>>(a, a_splits, stride, static_cast<const bf16*>(table),
+                                                       ids, ld, offset, static_cast<bf16*>(out), width, act);
   SHK_LAUNCH_CHECK("act_mul_rows");
   return 0;
 }

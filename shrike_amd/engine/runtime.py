@@ -69,7 +69,8 @@ class Runtime:
         [n, rows] in the compute dtype, or, where a matrix with few rows is split
         along k to fill the chip, the SplitSum of its parts.  reader "norm": the
         residual add of the next norm (no bias, width a multiple of 4 up to
-        8192); reader "position": the position-encoding and cache-write kernel."""
+        8192); reader "position": the position-encoding and cache-write kernel;
+        reader "rows": a kernel that adds the parts of any width (ops.act_mul_rows)."""
         n = x.shape[0]
         splits = ops.gemm_splits(n, w.rows, w.cols) if w.tiled is not None else 1
         if reader == "norm" and (bias is not None or w.rows % 4 or w.rows > 8192):

@@ -32,7 +32,7 @@ _SIGNATURES = {
     "shk_add_rows": [_P, _P, _P, _I, _I, _P],
     "shk_add_deltas": [_P, _P, _I, _P, _I, _P, _I, _I, _I, _P],
     "shk_add_normed_rmsnorm": [_P, _P, _I, _P, _F, _P, _F, _P, _I, _P, _I, _I, _I, _I, _P],
-    "shk_act_mul_rows": [_P, _P, _I, _P, c_longlong, _I, _I, _P, _I, _I, _I, _P],
+    "shk_act_mul_rows": [_P, _I, _P, _I, _P, c_longlong, _I, _I, _P, _I, _I, _I, _P],
     "shk_add_rmsnorm": [_P, _P, _P, _F, _P, _I, _P, _I, _I, _I, _I, _I, _P],
     "shk_act_mul": [_P, _P, _I, _I, _I, _I, _P],
     "shk_gemm": [_P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _I, _P],

@@ -187,15 +187,24 @@ def add_normed_rmsnorm(resid, delta, dweight, deps: float, weight=None, eps: flo
 
 def act_mul_rows(a, table, ids, offset: int, out, activation: str) -> None:
     """out[r, j] = act(a[r, j]) * table[ids[r], offset + j]: a gate times a slice of the
-    table row that the token chooses."""
+    table row that the token chooses.  `a` is a tensor of out's dtype or the SplitSum of
+    a product split along k."""
     n, width = out.shape
-    if a.shape != out.shape or not a.is_contiguous() or not out.is_contiguous() or a.dtype != out.dtype:
+    if not out.is_contiguous():
+        raise KernelError("act_mul_rows: out must be contiguous")
+    splits = 0
+    if isinstance(a, SplitSum):
+        if a.bias is not None or tuple(a.shape) != (n, width) or a.parts.dtype != torch.float32 \
+                or not a.parts.is_contiguous():
+            raise KernelError("act_mul_rows: partial sums must be contiguous float32 [splits, n, width] without a bias")
+        splits, a = a.parts.shape[0], a.parts
+    elif a.shape != out.shape or not a.is_contiguous() or a.dtype != out.dtype:
         raise KernelError("act_mul_rows: a and out must be contiguous, of one shape and dtype")
     if table.dim() != 2 or not table.is_contiguous() or table.dtype != out.dtype:
         raise KernelError("act_mul_rows: table must be a contiguous matrix of out's dtype")
     if offset < 0 or offset + width > table.shape[1] or ids.shape[0] < n:
         raise KernelError("act_mul_rows: the slice does not fit the table, or too few ids")
-    check(load().shk_act_mul_rows(_dev(a, "a"), _dev(table, "table"), dtype_code(out.dtype),
+    check(load().shk_act_mul_rows(_dev(a, "a"), splits, _dev(table, "table"), dtype_code(out.dtype),
                                   _dev(ids, "ids", torch.int32), table.shape[1], int(offset), table.shape[0],
                                   _dev(out, "out"), n, width, activation_code(activation), _stream()))
 

@@ -14,8 +14,9 @@ class TokenSide(SideInput):
 
     The table [vocab, slices * dim] is one tensor for all layers (its full name is
     in the spec); a layer reads its own slice of the token's row, whichever pass of
-    a loop it runs in.  The two products are ordinary products of the runtime; the
-    activation and the gather are one kernel; y stays pending with its norm, and
+    a loop it runs in.  The two products are ordinary products of the runtime (both
+    may come as partial sums of shares of k); the activation and the gather are one
+    kernel, which adds the first product's shares up; y stays pending with its norm, and
     the norm that follows (the next layer's, or the final one) forms
     resid + normed(y) and its own output in one pass over the row."""
 
@@ -43,14 +44,12 @@ class TokenSide(SideInput):
         self.w_proj = runtime.weight(tensors[self.tensor_name("proj")])
         self.weight = tensors[self.tensor_name("norm")]
         self.eps = float(s.eps)
-        self.linear = runtime.linear
         self.linear_deferred = runtime.linear_deferred
 
     def forward(self, ctx, hidden: HiddenState, x: torch.Tensor) -> None:
         s = self.spec
         n = x.shape[0]
-        gate = ctx.buffer("side_gate", (n, s.dim), ctx.dtype)
-        self.linear(x, self.w_gate, gate)
+        gate = self.linear_deferred(ctx, "side_gate", x, self.w_gate, reader="rows")
         gated = ctx.buffer("side_gated", (n, s.dim), ctx.dtype)
         ops.act_mul_rows(gate, self.table, ctx.token_ids, s.index * s.dim, gated, s.activation)
         hidden.pending = self.linear_deferred(ctx, "side_out", gated, self.w_proj)

@@ -37,15 +37,18 @@ def embed(tokens, table, scale):
     return table[tokens] * scale
 
 
-def rotate_interleaved(x, positions, base: float, dims: int):
+def rotate_interleaved(x, positions, base: float, dims: int, angle_dtype=None):
     """x [tokens, heads, dim].  Elements 2i and 2i+1 (i < dims/2) form a pair that
-    turns by positions * base**(-2i/dims); elements from `dims` on stay."""
+    turns by positions * base**(-2i/dims); elements from `dims` on stay.  The design
+    forms positions and angles in 32-bit: with angle_dtype=torch.float32 the rates are
+    rounded to it and the product is formed in it (thousands of radians are then known
+    to about 1e-4), otherwise everything has x's precision."""
     out = x.clone()
     if dims == 0:
         return out
-    i = torch.arange(dims // 2, dtype=x.dtype)
-    rate = base ** (-2.0 * i / dims)
-    angle = positions.to(x.dtype)[:, None] * rate[None, :]  # [tokens, dims/2]
+    i = torch.arange(dims // 2, dtype=torch.float64)
+    rate = (base ** (-2.0 * i / dims)).to(angle_dtype or x.dtype)
+    angle = (positions.to(rate.dtype)[:, None] * rate[None, :]).to(x.dtype)  # [tokens, dims/2]
     c, s = torch.cos(angle)[:, None, :], torch.sin(angle)[:, None, :]
     u, v = x[..., 0:dims:2], x[..., 1:dims:2]
     out[..., 0:dims:2] = u * c - v * s
@@ -146,3 +149,50 @@ def forward(cfg: dict, weights: dict, tokens, dtype=torch.float32, return_layers
     if return_layers:
         return logits, torch.stack(after)
     return logits
+
+
+def block_local_attention(q, k, v, scale: float, size: int, first: int = 0):
+    """q [n, heads, dim] at positions first .. first + n - 1 over keys and values
+    [ctx, groups, dim] at positions 0 .. ctx - 1: query i reads key j <= i of its own
+    block of `size` positions.  One query and one head at a time, written out."""
+    n, heads, dim = q.shape
+    groups = k.shape[1]
+    out = torch.zeros(n, heads, v.shape[2], dtype=q.dtype)
+    for r in range(n):
+        i = first + r
+        lo = i // size * size
+        for head in range(heads):
+            g = head // (heads // groups)
+            s = (k[lo : i + 1, g] @ q[r, head]) * scale
+            p = torch.softmax(s, dim=0)
+            out[r, head] = p @ v[lo : i + 1, g]
+    return out
+
+
+class PlainMofarax:
+    """A model folder read once; `logits(ids)` and greedy generation over it."""
+
+    def __init__(self, model_dir, dtype=torch.float64):
+        import json
+        from pathlib import Path
+
+        from safetensors.torch import load_file
+
+        self.cfg = json.loads((Path(model_dir) / "config.json").read_text())
+        self.weights = load_file(str(Path(model_dir) / "model.safetensors"))
+        self.dtype = dtype
+
+    def logits(self, token_ids, rows=None) -> torch.Tensor:
+        out = forward(self.cfg, self.weights, list(token_ids), self.dtype)
+        return out if rows is None else out[torch.tensor(list(rows), dtype=torch.long)]
+
+    def layers(self, token_ids) -> torch.Tensor:
+        return forward(self.cfg, self.weights, list(token_ids), self.dtype, return_layers=True)[1]
+
+    def greedy(self, prompt, max_new_tokens: int) -> list[int]:
+        seq, out = list(prompt), []
+        for _ in range(max_new_tokens):
+            tok = int(torch.argmax(self.logits(seq)[-1]))
+            out.append(tok)
+            seq.append(tok)
+        return out

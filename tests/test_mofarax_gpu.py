@@ -1,0 +1,239 @@
+"""The Mofarax decoder in the engine against its plain implementation
+(tests/plain/mofarax.py), on tiny models with random weights (tests/tiny_mofarax.py):
+the stream after every layer run; whole prompts, single tokens from the very first,
+portions down to two tokens and mixed batches over so few pages that they are used
+again (all pages that nobody holds poisoned with NaN); blocks of positions smaller
+than a page, beside page edges and larger than any sequence; long decoding across
+many block edges; greedy generation through the entry point and its scheduler."""
+
+import random
+
+import numpy as np
+import pytest
+import torch
+
+from .compare import GreedyCheck
+from .plain.mofarax import PlainMofarax
+from .tiny_mofarax import CONFIGS, PAGE_SIZES, make_model_dir
+from .traces import (TraceBuilder, changing_portions, check_pages, last_one_by_one, mixed, read_pages,
+                     run_trace, whole)
+
+pytestmark = pytest.mark.gpu
+
+TOL = {"float32": 1e-4, "bfloat16": 1.5e-2}
+# lengths that end before, on and after the edges of the models' blocks of positions
+# (24 and 40; 7; none; 33) and of their pages
+LENGTHS = {"P": [1, 9, 49, 97, 130, 24], "Q": [3, 15, 40, 29, 8], "R": [2, 70, 33, 100], "S": [5, 34, 67, 120, 33]}
+
+
+@pytest.fixture(scope="module")
+def model_root(tmp_path_factory):
+    return tmp_path_factory.mktemp("mofarax_models")
+
+
+def requests_for(name: str, lengths=None, seed: int = 0) -> dict[str, list[int]]:
+    rng = random.Random(sum(map(ord, name)) + seed)
+    vocab = CONFIGS[name]["vocab"]
+    return {f"r{i}": [rng.randrange(vocab) for _ in range(n)] for i, n in enumerate(lengths or LENGTHS[name])}
+
+
+def engine_parts(model_dir, dtype, page_size, pages, graphs=True):
+    from shrike_amd.cache import CacheManager
+    from shrike_amd.engine.loading import load_model
+    from shrike_amd.engine.runner import ModelRunner
+
+    model, rt, _cfg = load_model(model_dir, dtype)
+    cache = CacheManager(model.cache_specs(), page_size, pages, enable_prefix_caching=False)
+    cache.allocate(rt.dtype, rt.device)
+    return model, cache, ModelRunner(model, cache, rt, graphs=graphs)
+
+
+@pytest.mark.parametrize("name", ["P", "Q", "R", "S"])
+def test_the_stream_after_every_layer_run(name, model_root):
+    """float32: the residual stream after each run of a layer, loop passes included,
+    against the plain model's, for a prompt that crosses block edges."""
+    from shrike_amd.engine.runner import StepEntry
+
+    model_dir = make_model_dir(name, model_root, dtype="float32")
+    plain = PlainMofarax(model_dir)
+    ids = requests_for(name, [75])["r0"]
+    want = plain.layers(ids)
+    model, cache, runner = engine_parts(model_dir, "float32", 16, 16, graphs=False)
+    seen = []
+    for block in model.blocks:
+        def wrapped(ctx, hidden, layer_cache, inner=block.forward):
+            inner(ctx, hidden, layer_cache)
+            hidden.settle(ctx)
+            seen.append(hidden.resid.detach().cpu().double().clone())
+        block.forward = wrapped
+    seq = cache.new_sequence()
+    cache.append(seq, 0, len(ids))
+    runner.step([StepEntry(seq, ids, 0, [len(ids) - 1])])
+    assert len(seen) == want.shape[0] == len(model.spec.schedule)
+    for run, (got, ref) in enumerate(zip(seen, want)):
+        err = float((got - ref).abs().max() / ref.abs().max())
+        assert err <= 2e-5, f"layer run {run} (layer {model.spec.schedule[run].block}): rel err {err:.3e}"
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name, page_size", [("P", 16), ("Q", 4), ("Q", 16), ("R", 32), ("S", 16), ("P", 8)])
+def test_four_cuttings_agree_with_the_plain_implementation(name, page_size, dtype, model_root, tmp_path):
+    model_dir = make_model_dir(name, model_root, dtype=dtype)
+    vocab = CONFIGS[name]["vocab"]
+    seqs = requests_for(name)
+    plain = PlainMofarax(model_dir)
+    want = {rid: plain.logits(ids).numpy() for rid, ids in seqs.items()}
+
+    tb = TraceBuilder()
+    budget = max(-(-len(ids) // 64) * 64 for ids in seqs.values())
+    whole(tb, "w_", seqs)
+    last_one_by_one(tb, "d_", seqs, tail=45)
+    changing_portions(tb, "p_", seqs)
+    mixed_budget = budget + 128
+    mixed(tb, "m_", seqs, mixed_budget, seed=5)
+    outputs = run_trace(model_dir, dtype, tb.steps, mixed_budget, tmp_path / "out", vocab,
+                        block_size=page_size, poison=True, pages=True)
+    got = tb.collect(outputs)
+    assert all(np.isfinite(rows).all() for rows in outputs.values()), "a page that nobody holds was read"
+    reused = check_pages(tb.steps, read_pages(tmp_path / "out", tb.steps), page_size, mixed_budget // page_size)
+    assert reused > 0, "the pool was meant to be so small that pages are used again"
+
+    scale = {rid: np.abs(w).max() for rid, w in want.items()}
+    worst = {}
+    for (rid, pos), row in got.items():
+        cut, name_ = rid.split("_", 1)
+        err = np.abs(row.astype(np.float64) - want[name_][pos]).max() / scale[name_]
+        worst[cut] = max(worst.get(cut, 0.0), err)
+        assert err <= TOL[dtype], f"{rid} position {pos}: rel err {err:.3e}"
+    assert set(worst) == {"w", "d", "p", "m"}
+    for cut in "wdp":
+        assert all((f"{cut}_{rid}", p) in got for rid, ids in seqs.items() for p in range(len(ids)))
+    if dtype == "float32":  # the cuttings agree with each other more closely still
+        for (rid, pos), row in got.items():
+            cut, name_ = rid.split("_", 1)
+            assert np.abs(row - got[(f"w_{name_}", pos)]).max() / scale[name_] <= 1e-5
+    print(f"{name} page {page_size} {dtype}: worst rel err per cutting {worst}")
+
+
+@pytest.mark.parametrize("name", ["P", "Q", "S"])
+def test_long_decoding_from_the_first_token(name, model_root):
+    """Every token on the single-token path (graphs included), over many block
+    edges; pages that the blocks have passed are given back on the way, and what is
+    held never exceeds one block's pages plus the page being written."""
+    from shrike_amd.engine.runner import StepEntry
+
+    sizes = [layer["mixer"]["mask"]["size"] for layer in CONFIGS[name]["layers"]]
+    for dtype, tol in TOL.items():
+        model_dir = make_model_dir(name, model_root, dtype=dtype)
+        plain = PlainMofarax(model_dir)
+        page = PAGE_SIZES[name]
+        model, cache, runner = engine_parts(model_dir, dtype, page, 64)
+        ids = requests_for(name, [230], seed=3)["r0"]
+        want = plain.logits(ids)
+        seq = cache.new_sequence()
+        rows, most = [], 0
+        for p, tok in enumerate(ids):
+            cache.append(seq, p, 1)
+            rows.append(runner.step([StepEntry(seq, [tok], p, [0])]).cpu().clone())
+            cache.trim(seq, p + 1)
+            most = max(most, max(sum(x >= 0 for x in t) for t in seq.tables))
+        got = torch.cat(rows).double()
+        err = (got - want).abs().amax(-1) / want.abs().max()
+        if dtype == "bfloat16":
+            # Where a token's gates all come out near zero, the side input's norm divides a
+            # tiny vector by its own size, and the bfloat16 rounding of the gates' inputs
+            # (a few percent of such a gate) reaches the logits undamped: a few positions
+            # of 230 lie above the usual bound (narrow side inputs: 1 gate in 32 or 256).
+            assert float((err > tol).float().mean()) <= 0.05 and float(err.max()) <= 4 * tol, \
+                f"bfloat16: {int((err > tol).sum())} positions over {tol}, worst {float(err.max()):.3e}"
+        else:
+            assert float(err.max()) <= tol, f"{dtype}: worst at position {int(err.argmax())}: {float(err.max()):.3e}"
+        assert most <= -(-max(sizes) // page) + 1, "pages behind the current block were kept"
+        assert runner.graph_replays > 100
+        cache.free(seq)
+        cache.check([])
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name, lengths, new, budget", [("P", [1, 20, 47, 30], 60, 16), ("Q", [5, 13, 2], 30, 512),
+                                                        ("R", [40, 3], 25, 24), ("S", [31, 66, 8], 70, 32)])
+def test_greedy_generation_through_the_entry_point(name, lengths, new, budget, dtype, model_root):
+    """Prompts in portions under a small token budget beside decoding requests, through
+    LLM.generate and its scheduler; float32: the plain model's greedy tokens exactly."""
+    from shrike_amd import LLM, SamplingParams
+
+    model_dir = make_model_dir(name, model_root, dtype=dtype)
+    plain = PlainMofarax(model_dir)
+    prompts = list(requests_for(name, lengths, seed=9).values())
+    llm = LLM(str(model_dir), dtype=dtype, block_size=PAGE_SIZES[name], num_kv_blocks=96, max_tokens_per_step=budget)
+    outs = llm.generate(prompts, SamplingParams(max_new_tokens=new, ignore_eos=True))
+    assert [len(o) for o in outs] == [new] * len(prompts)
+    check = GreedyCheck(plain, dtype)
+    for prompt, out in zip(prompts, outs):
+        check.request(prompt, out)
+    check.finish()
+    assert llm.engine.cache.num_free == llm.engine.cache.num_pages
+    assert llm.engine.cache.slots.num_free == llm.engine.cache.slots.num_slots
+
+
+def test_generation_survives_preemption_when_pages_run_out(model_root):
+    """So few pages that the newest request is preempted and recomputes: the tokens
+    are the plain model's all the same."""
+    from shrike_amd import LLM, SamplingParams
+
+    model_dir = make_model_dir("R", model_root, dtype="float32")  # no block bound: nothing is given back early
+    plain = PlainMofarax(model_dir)
+    prompts = list(requests_for("R", [30, 28, 33], seed=2).values())
+    llm = LLM(str(model_dir), dtype="float32", block_size=16, num_kv_blocks=9, max_tokens_per_step=64)
+    outs = llm.generate(prompts, SamplingParams(max_new_tokens=40, ignore_eos=True))
+    assert llm.engine.metrics()["preemptions"] > 0
+    for prompt, out in zip(prompts, outs):
+        assert out == plain.greedy(prompt, 40)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_graphs_and_recorded_launches_equal_kernel_by_kernel_steps(dtype, model_root):
+    """The same steps with and without HIP graphs and recorded launch lists: the
+    same bits."""
+    from shrike_amd.engine.runner import StepEntry
+
+    model_dir = make_model_dir("P", model_root, dtype=dtype)
+    ids = requests_for("P", [90, 41], seed=4)
+    results = []
+    for graphs in (True, False):
+        model, cache, runner = engine_parts(model_dir, dtype, 16, 32, graphs=graphs)
+        a, b = cache.new_sequence(), cache.new_sequence()
+        rows = []
+        pa = pb = 0
+        for step in range(40):
+            entries = []
+            na = 7 if pa < 60 else 1  # portions of a first, then single tokens
+            na = min(na, len(ids["r0"]) - pa)
+            if na:
+                cache.append(a, pa, na)
+                entries.append(StepEntry(a, ids["r0"][pa : pa + na], pa, [na - 1]))
+            nb = 1 if pb < len(ids["r1"]) else 0
+            if nb:
+                cache.append(b, pb, 1)
+                entries.append(StepEntry(b, [ids["r1"][pb]], pb, [0]))
+            if not entries:
+                break
+            rows.append(runner.step(entries).cpu().clone())
+            pa, pb = pa + na, pb + nb
+            cache.trim(a, pa), cache.trim(b, pb)
+        if graphs:
+            assert runner.graph_replays > 0 and runner.list_replays > 0
+        results.append(torch.cat(rows))
+    assert torch.equal(results[0], results[1])
+
+
+def test_command_line_generates_with_a_model_folder(model_root, capsys):
+    from shrike_amd.__main__ import main
+
+    model_dir = make_model_dir("Q", model_root, dtype="float32")
+    rc = main(["--model", str(model_dir), "--prompt-ids", "5,6,7,8,300,2", "--max-tokens", "9", "--dtype", "fp32",
+               "--block-size", "4", "--num-kv-blocks", "16", "--ignore-eos", "--metrics"])
+    assert rc == 0
+    out = capsys.readouterr()
+    assert [int(t) for t in out.out.split()] == PlainMofarax(model_dir).greedy([5, 6, 7, 8, 300, 2], 9)
+    assert "tokens_generated" in out.err
