@@ -10,9 +10,9 @@ import torch
 import torch.nn.functional as F
 
 from shrike_amd.cache import CacheManager
-from shrike_amd.config.registry import ConfigError, architecture_name, get_architecture
+from shrike_amd.config import registry  # (names through the modules: another test reloads them)
 from shrike_amd.models import DecoderModel
-from shrike_amd.models.mofarax import MofaraxConfig, build_spec, layer_schedule
+from shrike_amd.models import mofarax as mof
 
 from .plain import mofarax as plain
 from .tiny_mofarax import CONFIGS, MOF_P, MOF_R
@@ -23,10 +23,10 @@ from .tiny_mofarax import CONFIGS, MOF_P, MOF_R
 @pytest.mark.parametrize("name", sorted(CONFIGS))
 def test_config_reads_back(name):
     raw = CONFIGS[name]
-    assert architecture_name(raw) == "Mofarax"
-    arch = get_architecture("Mofarax")
+    assert registry.architecture_name(raw) == "Mofarax"
+    arch = registry.get_architecture("Mofarax")
     cfg = arch.config_cls.from_dict(raw)
-    assert MofaraxConfig.from_dict(cfg.to_dict()) == cfg
+    assert arch.config_cls.from_dict(cfg.to_dict()) == cfg
     assert len(cfg.layers) == len(raw["layers"])
     assert cfg.layers[0].mixer.mask_size == raw["layers"][0]["mixer"]["mask"]["size"]
     assert cfg.embedding_scale == raw["embedding"]["scale"]
@@ -47,12 +47,12 @@ def test_config_reads_back(name):
 def test_config_refuses_what_it_cannot_run(change, message):
     raw = copy.deepcopy(MOF_P)
     change(raw)
-    with pytest.raises(ConfigError, match=message):
-        MofaraxConfig.from_dict(raw)
+    with pytest.raises(registry.ConfigError, match=message):
+        mof.MofaraxConfig.from_dict(raw)
 
 
 def test_tensors_the_model_declares():
-    model = DecoderModel(build_spec(MofaraxConfig.from_dict(MOF_P)))
+    model = DecoderModel(mof.build_spec(mof.MofaraxConfig.from_dict(MOF_P)))
     shapes = {p.name: tuple(p.shape) for p in model.params()}
     assert shapes["embed"] == (199, 64) and shapes["head"] == (199, 64) and shapes["final.norm"] == (64,)
     assert shapes["loop.step"] == (3, 64)
@@ -63,21 +63,21 @@ def test_tensors_the_model_declares():
     assert not any(n.startswith("l1.mlp") for n in shapes)  # a layer without a feed-forward
     assert not any(".v" in n for n in shapes)  # no value projection anywhere
     assert shapes["l1.side.gate"] == (8, 64) and shapes["l1.side.proj"] == (64, 8) and shapes["l1.side.norm"] == (64,)
-    plain_model = DecoderModel(build_spec(MofaraxConfig.from_dict(MOF_R)))
+    plain_model = DecoderModel(mof.build_spec(mof.MofaraxConfig.from_dict(MOF_R)))
     names = {p.name for p in plain_model.params()}
     assert "loop.step" not in names and "side.embed" not in names and not any(".side." in n for n in names)
 
 
 def test_schedule_of_a_loop():
-    runs = layer_schedule(5, (1, 3, 3))
+    runs = mof.layer_schedule(5, (1, 3, 3))
     assert [e.block for e in runs] == [0, 1, 2, 1, 2, 1, 2, 3, 4]
     assert [e.add_embedding for e in runs] == [False, False, False, True, False, True, False, False, False]
     assert [e.add_vector for e in runs] == [None, ("loop.step", 0), None, ("loop.step", 1), None, ("loop.step", 2),
                                             None, None, None]
     assert all(e.cache_of is None for e in runs)  # every pass has caches of its own
-    once = layer_schedule(3, (0, 3, 1))
+    once = mof.layer_schedule(3, (0, 3, 1))
     assert [e.add_vector for e in once] == [("loop.step", 0), None, None] and not any(e.add_embedding for e in once)
-    assert [(e.block, e.add_vector) for e in layer_schedule(2, None)] == [(0, None), (1, None)]
+    assert [(e.block, e.add_vector) for e in mof.layer_schedule(2, None)] == [(0, None), (1, None)]
     assert plain.layer_runs({"layers": [0] * 5, "loop": {"start": 1, "stop": 3, "times": 3}}) == [
         (0, None), (1, 0), (2, None), (1, 1), (2, None), (1, 2), (2, None), (3, None), (4, None)]
 
@@ -85,7 +85,7 @@ def test_schedule_of_a_loop():
 # ------------------------------------------------------------------ cache manager
 
 def test_pages_behind_the_current_block_are_given_back():
-    model = DecoderModel(build_spec(MofaraxConfig.from_dict(MOF_P)))
+    model = DecoderModel(mof.build_spec(mof.MofaraxConfig.from_dict(MOF_P)))
     specs = model.cache_specs()
     assert len(specs) == 1 + 2 * 3 and all(s is not None for s in specs)
     cache = CacheManager(specs, 8, 40, enable_prefix_caching=False)

@@ -63,6 +63,7 @@ def test_rope_frequencies_are_a_geometric_sequence_from_one_down():
 
 
 def test_rope_scores_depend_only_on_distance():
+    torch.manual_seed(0)  # (the float32 angle tables leave differences of some 1e-6, whatever ran before)
     d, theta = 32, 1e6
     q, k = torch.randn(1, 1, d, dtype=torch.float64), torch.randn(1, 1, d, dtype=torch.float64)
 
