@@ -413,6 +413,8 @@ def run_designs(args, qcfg) -> dict:
     mcfg, msizes = mofarax_like(qcfg, args.mask_size, args.side_dim)
     out = {}
     for name, spec, sizes in (("qwen2", qwen2.build_spec(qcfg), qcfg), ("mofarax", mofarax.build_spec(mcfg), msizes)):
+        if args.design_only and name != args.design_only:
+            continue
         engine = make_engine(sizes, spec, 64, args.seed)
         rng = random.Random(args.seed + 5)
 
@@ -583,6 +585,8 @@ def main() -> int:
     ap.add_argument("--mofarax", action="store_true",
                     help="instead of the default run: the Mofarax design beside Qwen2 at the layer sizes of "
                          "--shape, random weights: prompt, decode at batch 1 / 8 / 64, per-kernel times")
+    ap.add_argument("--design-only", choices=["qwen2", "mofarax"], default=None,
+                    help="--mofarax: run only this one of the two (for a profile of one model's kernels)")
     ap.add_argument("--mask-size", type=int, default=8192, metavar="N",
                     help="--mofarax: positions per block of its attention (8192: no fewer keys than Qwen2 reads)")
     ap.add_argument("--side-dim", type=int, default=256, metavar="N", help="--mofarax: width of its per-layer token input")
@@ -620,7 +624,7 @@ def main() -> int:
         print(json.dumps({
             "metric": f"Mofarax beside Qwen2 at the Qwen2.5-{args.shape.upper()} layer sizes: prompt tok/s, decode "
                       "tok/s, us per kernel",
-            "value": designs["mofarax"]["decode_b8"]["tok_s"], "unit": "tok/s", "n_gpus": 1, "higher_is_better": True,
+            "value": designs[args.design_only or "mofarax"]["decode_b8"]["tok_s"], "unit": "tok/s", "n_gpus": 1, "higher_is_better": True,
             "dtype": "bf16", "data": "synthetic: random weights, prompt ids uniform in [0, vocab)",
             "config": {"shape": args.shape, "layers": cfg.num_hidden_layers, "mask_size": args.mask_size,
                        "side_dim": args.side_dim, "prompt": PROMPT_LEN, "decode_steps": args.design_steps},

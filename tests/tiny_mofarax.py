@@ -5,7 +5,8 @@ heads rotated whole, in part and not at all, blocks of positions smaller than a
 page, beside a page's edge, just over 32 and larger than any test sequence,
 layers without a feed-forward, layers that differ within one model (two page
 groups), loops that start after the first layer, run once, twice or three
-times, or are absent, a side input of odd width or none."""
+times, or are absent, a side input of odd width or none; one model whose sizes are
+multiples of nothing, with blocks of a single position in one layer."""
 
 from __future__ import annotations
 
@@ -55,9 +56,18 @@ MOF_S = {
                _layer(_mixer(2, 1, 96, 33, 96, base=2.0e5), None)],
 }
 
-CONFIGS = {"P": MOF_P, "Q": MOF_Q, "R": MOF_R, "S": MOF_S}
-SEEDS = {"P": 5, "Q": 17, "R": 29, "S": 43}
-PAGE_SIZES = {"P": 16, "Q": 4, "R": 32, "S": 16}
+# sizes that are multiples of nothing: rows that no vector load takes, a head of 10
+MOF_T = {
+    "architecture": "Mofarax", "vocab": 97, "width": 100,
+    "embedding": {"scale": 2.25}, "norm": {"eps": 1e-4}, "token_side": {"dim": 3},
+    "loop": {"start": 1, "stop": 2, "times": 2},
+    "layers": [_layer(_mixer(2, 2, 10, 5, 6, base=90.0, scale=0.4), 52), _layer(_mixer(6, 2, 10, 1, 10, base=90.0), 30),
+               _layer(_mixer(2, 1, 10, 11, 2, base=4.0), None)],
+}
+
+CONFIGS = {"P": MOF_P, "Q": MOF_Q, "R": MOF_R, "S": MOF_S, "T": MOF_T}
+SEEDS = {"P": 5, "Q": 17, "R": 29, "S": 43, "T": 59}
+PAGE_SIZES = {"P": 16, "Q": 4, "R": 32, "S": 16, "T": 8}
 
 
 def make_model_dir(name: str, root=None, dtype: str = "float32", mode: str = "unit") -> Path:
