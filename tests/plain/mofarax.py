@@ -151,16 +151,19 @@ def forward(cfg: dict, weights: dict, tokens, dtype=torch.float32, return_layers
     return logits
 
 
-def block_local_attention(q, k, v, scale: float, size: int, first: int = 0):
+def block_local_attention(q, k, v, scale: float, size: int, first: int = 0, window: int | None = None):
     """q [n, heads, dim] at positions first .. first + n - 1 over keys and values
     [ctx, groups, dim] at positions 0 .. ctx - 1: query i reads key j <= i of its own
-    block of `size` positions.  One query and one head at a time, written out."""
+    block of `size` positions (and, with a window, only the last `window` keys up to
+    i).  One query and one head at a time, written out."""
     n, heads, dim = q.shape
     groups = k.shape[1]
     out = torch.zeros(n, heads, v.shape[2], dtype=q.dtype)
     for r in range(n):
         i = first + r
         lo = i // size * size
+        if window is not None:
+            lo = max(lo, i - window + 1)
         for head in range(heads):
             g = head // (heads // groups)
             s = (k[lo : i + 1, g] @ q[r, head]) * scale

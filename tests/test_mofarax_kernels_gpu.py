@@ -97,7 +97,7 @@ def standing_out(ctx, heads, kv_heads, head_dim, target, seed):
 
 
 def run_attention(ops, kind, q, positions, tables, k_pool, v_pool, heads, kv_heads, head_dim, page_size, chunk, scale,
-                  q_lens, starts):
+                  q_lens, starts, window=None):
     """One of the attention kernels on a step of len(q_lens) sequences (single tokens
     for "decode")."""
     n = q.shape[0]
@@ -108,12 +108,12 @@ def run_attention(ops, kind, q, positions, tables, k_pool, v_pool, heads, kv_hea
     token_seq = i32([s for s, l in enumerate(q_lens) for _ in range(l)])
     if kind == "general":
         ops.attention(qd, out, heads, kv_heads, head_dim, i32(positions), token_seq, tables, k_pool, v_pool,
-                      page_size, None, scale, chunk=chunk)
+                      page_size, window, scale, chunk=chunk)
     elif kind == "decode":
         nsplit = 3
         partial = torch.full((n * heads * nsplit * (head_dim + 2),), float("nan"), device="cuda")
         ops.attention_decode(qd, out, n, heads, kv_heads, head_dim, i32(positions), tables, k_pool, v_pool,
-                             page_size, None, scale, partial, nsplit, chunk=chunk)
+                             page_size, window, scale, partial, nsplit, chunk=chunk)
     else:
         cu = [0]
         for l in q_lens:
@@ -124,7 +124,7 @@ def run_attention(ops, kind, q, positions, tables, k_pool, v_pool, heads, kv_hea
         wg_q0 = [q0 for l in q_lens for q0 in range(0, l, run)]
         launch = ops.attention_prefill_shared if kind == "shared" else ops.attention_prefill
         launch(qd, out, len(wg_seq), heads, kv_heads, head_dim, i32(cu), i32(ctx), i32(wg_seq), i32(wg_q0), tables,
-               k_pool, v_pool, page_size, None, scale, chunk=chunk)
+               k_pool, v_pool, page_size, window, scale, chunk=chunk)
     return out.view(n, heads, head_dim)
 
 
@@ -167,9 +167,11 @@ def test_a_key_just_inside_and_just_outside_the_block(ops, kind, dtype, chunk, c
             assert near > 0.3, "a key before the block's first position was read"
 
 
+@pytest.mark.parametrize("window", [None, 25])
 @pytest.mark.parametrize("kind, dtype", KINDS)
-def test_block_local_attention_on_a_mixed_batch(ops, kind, dtype):
-    """Several sequences at once, contexts before, on and after block and page edges."""
+def test_block_local_attention_on_a_mixed_batch(ops, kind, dtype, window):
+    """Several sequences at once, contexts before, on and after block and page edges;
+    also with a window beside the block: the later of the two first keys holds."""
     torch.manual_seed(21)
     heads, kv_heads, head_dim, page_size, chunk = 6, 3, 32, 16, 40
     if kind in ("decode", "general"):
@@ -188,12 +190,12 @@ def test_block_local_attention_on_a_mixed_batch(ops, kind, dtype):
     positions = [p for s, l in zip(starts, q_lens) for p in range(s, s + l)]
     scale = 0.9 * head_dim**-0.5
     got = run_attention(ops, kind, q, positions, tables, k_pool, v_pool, heads, kv_heads, head_dim, page_size, chunk,
-                        scale, q_lens, starts)
+                        scale, q_lens, starts, window=window)
     assert not torch.isnan(got.float()).any(), "a slot outside the context was read"
     off = 0
     for s, l in enumerate(q_lens):
         want = plain.block_local_attention(q[off : off + l].to(dtype).double(), keys[s].to(dtype).double(),
-                                           values[s].to(dtype).double(), scale, chunk, first=starts[s])
+                                           values[s].to(dtype).double(), scale, chunk, first=starts[s], window=window)
         close(got[off : off + l], want, dtype, scale=1.0)
         off += l
 
