@@ -64,13 +64,17 @@ class Runtime:
         else:
             ops.gemm(x, w.dense, out, bias=bias, accumulate=accumulate)
 
-    def linear_deferred(self, ctx, name: str, x, w: LinearWeight, bias=None, reader="norm"):
+    def linear_deferred(self, ctx, name: str, x, w: LinearWeight, bias=None, reader="norm",
+                        keep_float32: bool = False):
         """x @ w.T + bias for a reader that can add up partial sums: a tensor
         [n, rows] in the compute dtype, or, where a matrix with few rows is split
         along k to fill the chip, the SplitSum of its parts.  reader "norm": the
         residual add of the next norm (no bias, width a multiple of 4 up to
         8192); reader "position": the position-encoding and cache-write kernel;
-        reader "rows": a kernel that adds the parts of any width (ops.act_mul_rows)."""
+        reader "rows": a kernel that adds the parts of any width (ops.act_mul_rows).
+        keep_float32: a product that is not split comes as a SplitSum of one float32
+        part instead of a tensor in the compute dtype (for a reader that takes parts
+        and is sensitive to the rounding of its input)."""
         n = x.shape[0]
         splits = ops.gemm_splits(n, w.rows, w.cols) if w.tiled is not None else 1
         if reader == "norm" and (bias is not None or w.rows % 4 or w.rows > 8192):
@@ -79,6 +83,10 @@ class Runtime:
             parts = ctx.buffer(name + "_parts", (splits, n, w.rows), torch.float32)
             ops.gemm_tiled_weight(x, w.tiled, w.rows, w.cols, parts, splits=splits)
             return ops.SplitSum(parts, bias)
+        if keep_float32 and self.dtype != torch.float32:
+            parts = ctx.buffer(name + "_parts", (1, n, w.rows), torch.float32)
+            self.linear(x, w, parts[0], bias=bias)
+            return ops.SplitSum(parts)
         out = ctx.buffer(name, (n, w.rows), self.dtype)
         self.linear(x, w, out, bias=bias)
         return out

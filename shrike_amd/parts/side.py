@@ -16,7 +16,9 @@ class TokenSide(SideInput):
     in the spec); a layer reads its own slice of the token's row, whichever pass of
     a loop it runs in.  The two products are ordinary products of the runtime (both
     may come as partial sums of shares of k); the activation and the gather are one
-    kernel, which adds the first product's shares up; y stays pending with its norm, and
+    kernel, which adds the first product's shares up (the gates reach it in float32,
+    split or not: a gate that is rounded to 8 bits first loses more where gelu is
+    steep, and the norm below does not damp what a tiny y has lost); y stays pending with its norm, and
     the norm that follows (the next layer's, or the final one) forms
     resid + normed(y) and its own output in one pass over the row."""
 
@@ -49,7 +51,7 @@ class TokenSide(SideInput):
     def forward(self, ctx, hidden: HiddenState, x: torch.Tensor) -> None:
         s = self.spec
         n = x.shape[0]
-        gate = self.linear_deferred(ctx, "side_gate", x, self.w_gate, reader="rows")
+        gate = self.linear_deferred(ctx, "side_gate", x, self.w_gate, reader="rows", keep_float32=True)
         gated = ctx.buffer("side_gated", (n, s.dim), ctx.dtype)
         ops.act_mul_rows(gate, self.table, ctx.token_ids, s.index * s.dim, gated, s.activation)
         hidden.pending = self.linear_deferred(ctx, "side_out", gated, self.w_proj)
