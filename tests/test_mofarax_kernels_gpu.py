@@ -133,7 +133,8 @@ KINDS = [("general", torch.float32), ("general", torch.bfloat16), ("decode", tor
 
 
 @pytest.mark.parametrize("kind, dtype", KINDS)
-@pytest.mark.parametrize("chunk, ctx", [(48, 150), (33, 100), (16, 65), (7, 40), (1, 9), (500, 700), (120, 361)])
+@pytest.mark.parametrize("chunk, ctx", [(48, 150), (33, 100), (16, 65), (7, 40), (1, 9), (500, 700), (120, 361),
+                                        (4096, 1500)])  # the last: one block, the key 1,499 positions back
 def test_a_key_just_inside_and_just_outside_the_block(ops, kind, dtype, chunk, ctx):
     """The last query's block starts at `first`.  A key that stands out at `first` is
     all the query sees; the same key one position earlier (the last of the block
@@ -145,7 +146,7 @@ def test_a_key_just_inside_and_just_outside_the_block(ops, kind, dtype, chunk, c
         if target < 0:
             continue
         q, k, v = standing_out(ctx, heads, kv_heads, head_dim, target, seed=ctx + target)
-        tables, k_pool, v_pool = paged_setup([ctx], page_size, 64, kv_heads, head_dim, dtype, seed=1)
+        tables, k_pool, v_pool = paged_setup([ctx], page_size, 128, kv_heads, head_dim, dtype, seed=1)
         fill_pools_from(tables, k_pool, v_pool, 0, k, v, page_size)
         if kind == "decode" or kind == "general":
             got = run_attention(ops, kind, q, [pos], tables, k_pool, v_pool, heads, kv_heads, head_dim, page_size,
