@@ -60,6 +60,13 @@ class AttentionSpec:
     applied to queries and keys after the projections; None leaves them as they
     are.  ``values_from_keys``: there is no value projection; a token's values are
     its keys as projected, before ``position`` is applied.
+    ``value_dim``: size of a head's value where it differs from ``head_dim`` (the
+    size of queries and keys).  ``softcap``: scaled scores become cap * tanh(score /
+    cap).  ``sinks``: a learned number per query head whose exponential joins the
+    softmax's denominator; it has no key and no value.  ``query_temperature`` =
+    (coef, every): the queries at position p are multiplied by 1 + coef *
+    ln(floor((p + 1) / every) + 1).  ``value_norm_eps``: each head's value is divided
+    by sqrt(mean(v^2) + eps), without a weight, before it is cached.
     """
 
     kind: ClassVar[str] = "paged_attention"
@@ -73,6 +80,74 @@ class AttentionSpec:
     position: object = None
     chunk: int | None = None
     values_from_keys: bool = False
+    names: Names = ()
+    value_dim: int | None = None
+    softcap: float | None = None
+    sinks: bool = False
+    query_temperature: tuple | None = None
+    value_norm_eps: float | None = None
+
+
+@dataclass(frozen=True)
+class LatentAttentionSpec:
+    """Attention whose queries, keys and values come through low-rank latents.
+
+    c_q = norm(W_dq x) (q_rank), q = W_uq c_q: per head ``head_dim`` unrotated and
+    ``rot_dim`` rotated elements.  W_dkv x has kv_rank + rot_dim rows: the first
+    kv_rank, normed, are the key/value latent c; the rest, not normed, are one rotated
+    key part that all heads share.  Per head the unrotated key is W_uk c and the value
+    W_uv c (``value_dim``); score = (q_plain . k_plain + q_rot . k_rot) * scale.  The
+    rotation turns neighbouring pairs (2i, 2i + 1) of the rotated part by position *
+    rot_theta ** (-2i / rotated), for the first ``rotated`` elements of the part (None: all
+    of it; the rest pass unchanged).  Both norms are RMS norms with a weight and ``eps``.
+    ``window`` / ``chunk`` bound the keys as in AttentionSpec.  Only c and the rotated key
+    part are cached."""
+
+    kind: ClassVar[str] = "latent_attention"
+    num_heads: int
+    head_dim: int
+    rot_dim: int
+    value_dim: int
+    q_rank: int
+    kv_rank: int
+    scale: float
+    eps: float
+    rot_theta: float = 10000.0
+    window: int | None = None
+    chunk: int | None = None
+    names: Names = ()
+    rotated: int | None = None
+
+
+@dataclass(frozen=True)
+class MLSTMSpec:
+    """A matrix memory with exponential gates (the mLSTM of xLSTM).  Per head: q = W_q x *
+    head_dim ** -0.5, k = W_k x, v = W_v x (``value_dim``); log gates i = cap tanh((W_i x
+    + b_i) / cap), f = logsigmoid(cap tanh((W_f x + b_f) / cap)); state S [head_dim,
+    value_dim], n [head_dim], running maximum m (all zero before the first token):
+        m' = max(f + m, i);  S' = exp(f + m - m') S + exp(i - m') k v^T;  n' likewise with k;
+        o = S'^T q / (max(|n' . q|, exp(-m')) + 1e-6).
+    Each head's o is divided by its root mean square (``eps``), the heads side by side are
+    multiplied by a weight and by sigmoid(W_g x), then W_o."""
+
+    kind: ClassVar[str] = "mlstm"
+    num_heads: int
+    head_dim: int
+    value_dim: int
+    gate_cap: float
+    eps: float
+    names: Names = ()
+
+
+@dataclass(frozen=True)
+class DenseFFNSpec:
+    """down(act(up(x))) without biases.  ``activation`` "xielu": for z > 0, softplus(p) z^2
+    + z / 2; else (1/2 + softplus(q)) (exp(z) - 1 - z) + z / 2, with the layer's own two
+    numbers (p, q) in a tensor of two elements."""
+
+    kind: ClassVar[str] = "dense_act"
+    intermediate_size: int
+    activation: str = "xielu"
     names: Names = ()
 
 
@@ -107,7 +182,8 @@ class TokenSideSpec:
 
 @dataclass(frozen=True)
 class BlockSpec:
-    """x += mixer(mixer_norm(x)); x += ffn(ffn_norm(x)).
+    """x += mixer(mixer_norm(x)); x += ffn(ffn_norm(x)).  ``ffn`` may be None: the
+    layer then has no feed-forward and no second norm.
 
     ``name`` is the prefix of the block's tensors in the weight file; the
     ``*_name`` fields are the sub-names of its parts below that prefix.
@@ -149,6 +225,21 @@ class TokenEmbeddingSpec:
     kind: ClassVar[str] = "token_lookup"
     vocab_size: int
     scale: float = 1.0
+    names: Names = ()
+
+
+@dataclass(frozen=True)
+class PairHashEmbeddingSpec:
+    """x = table[token] + pairs[(previous token * mul_prev + token * mul_cur) mod buckets];
+    a sequence's first token, which has no previous one, takes row `buckets` (the last of
+    the buckets + 1 rows).  ``pair_name`` is the full name of the pair table."""
+
+    kind: ClassVar[str] = "token_pair_hash"
+    vocab_size: int
+    buckets: int
+    mul_prev: int
+    mul_cur: int
+    pair_name: str = "bigram"
     names: Names = ()
 
 

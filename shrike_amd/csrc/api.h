@@ -145,12 +145,26 @@ int shk_rope_kv_store(void* qkv, int dtype, int n, int heads, int kv_heads, int 
 // when window <= 0) through tables[s]; with chunk > 0 only those of them that lie
 // in p's own block of `chunk` positions, floor(j / chunk) == floor(p / chunk) (the
 // same two bounds in every attention launcher below).  q has row stride q_stride elements,
-// out is [n, heads * head_dim].  Softmax and accumulation are float32.
+// out is [n, heads * v_dim].  Softmax and accumulation are float32.  v_dim is the size of
+// a value (the value pool is [num_pages, kv_heads, v_dim, page_size]); softcap > 0 caps
+// the scaled scores, s <- softcap * tanh(s / softcap); sinks (float32 [heads] or null)
+// adds exp(sinks[head]) to the softmax's denominator, a term without key or value.
 int shk_attention(const void* q, int q_stride, void* out, int dtype, int n, int heads,
                   int kv_heads, int head_dim, const int32_t* positions, const int32_t* token_seq,
                   const int32_t* tables, int table_stride, int num_seqs, const void* k_pool,
                   const void* v_pool, int page_size, int num_pages, int window, int chunk, float scale,
-                  void* stream);
+                  int v_dim, float softcap, const float* sinks, void* stream);
+
+// Cache write for attention without rotation.  qkv is [n, heads * head_dim + kv_heads *
+// (head_dim + v_dim)]: queries, keys, values.  q_every > 0: the queries of the token at
+// position p are multiplied by 1 + q_coef * ln(floor((p + 1) / q_every) + 1), in place.
+// v_eps > 0: each head's value is divided by sqrt(mean(v^2) + v_eps) before it is stored.
+// Keys and values go to their page slots in the layouts of shk_rope_kv_store (values
+// [num_pages, kv_heads, v_dim, page_size]); write_kv 0 leaves the pools alone.
+int shk_qkv_store(void* qkv, int dtype, int n, int heads, int kv_heads, int head_dim, int v_dim,
+                  float q_coef, int q_every, float v_eps, const int32_t* positions,
+                  const int32_t* token_seq, const int32_t* tables, int table_stride, void* k_pool,
+                  void* v_pool, int page_size, int num_pages, int write_kv, void* stream);
 
 // 1 if the MFMA attention kernels take these shapes (head_dim a multiple of 32
 // up to 256, page_size a multiple of 16, at most 16 query heads per key/value
@@ -200,6 +214,68 @@ int shk_attention_prefill_shared_bf16(const void* q, int q_stride, void* out, in
                                       int page_size, int window, int chunk, float scale, int small,
                                       float* partial, int nsplit, int first_token,
                                       int prompt_tokens, void* stream);
+
+// Attention through latents (latent.hip).  shk_latent_prepare: `down` is [n, q_rank +
+// kv_rank + rot_dim], a token's joint down-projection; q_latent [n, q_rank] receives
+// down[:, :q_rank] * rsqrt(mean^2 + eps) * q_weight; the token's row of `pool`
+// ([num_pages, page_size, kv_rank + rot_dim], page through tables as elsewhere) receives
+// the next kv_rank columns normed likewise with kv_weight, then the last rot_dim columns
+// with neighbouring pairs (2i, 2i + 1) turned by position * inv_freq[i].
+int shk_latent_prepare(const void* down, int dtype, int n, int q_rank, int kv_rank, int rot_dim,
+                       const float* q_weight, const float* kv_weight, float eps, const float* inv_freq,
+                       const int32_t* positions, const int32_t* token_seq, const int32_t* tables,
+                       int table_stride, void* q_latent, void* pool, int page_size, int num_pages,
+                       int write_kv, void* stream);
+// dst[t, h * dst_head + dst_off + e] = the rotation of src[t, h * src_head + src_off + e],
+// e < rot_dim, pairs (2i, 2i + 1) turned by positions[t] * inv_freq[i]; rows src_row /
+// dst_row elements apart.
+int shk_rotate_heads(const void* src, int src_row, int src_head, int src_off, void* dst, int dst_row,
+                     int dst_head, int dst_off, int dtype, int n, int heads, int rot_dim,
+                     const float* inv_freq, const int32_t* positions, void* stream);
+// q [n, heads, key_dim], out [n, heads, v_dim]: every head attends over the rows of the
+// token's sequence in `pool` ([num_pages, page_size, key_dim]); score = q . row * scale, the
+// values are the rows' first v_dim elements.  window / chunk as in shk_attention.
+int shk_latent_attention(const void* q, void* out, int dtype, int n, int heads, int key_dim, int v_dim,
+                         const int32_t* positions, const int32_t* token_seq, const int32_t* tables,
+                         int table_stride, const void* pool, int page_size, int num_pages, int window,
+                         int chunk, float scale, void* stream);
+
+// A batch of products of one shape: out_b[n, m] = a_b[n, k] @ w_b[m, k]^T for b < batch, with
+// a_b = a + b * a_batch (rows lda apart), w_b = w + b * w_batch (contiguous), out_b = out + b *
+// out_batch (rows ldo apart); all of `dtype`, float32 accumulation in ascending k.
+int shk_gemm_batched(const void* a, const void* w, void* out, int n, int m, int k, int lda, int ldo,
+                     int batch, long long a_batch, long long w_batch, long long out_batch, int dtype,
+                     void* stream);
+
+// The mLSTM recurrence (mlstm.hip) for the tokens of a step.  proj [n, ld] float32 holds each
+// token's projections: queries at column q_off ([heads, dim]), keys at k_off, values at v_off
+// ([heads, v_dim]), the input and forget gates' pre-activations at i_off and f_off ([heads]);
+// i_bias / f_bias [heads] are added; cap bounds the gates; queries are multiplied by q_scale.
+// Sequence s owns rows cu_q[s] .. cu_q[s + 1]; its state lies at state + slots[s] *
+// slot_stride (shk_mlstm_state_floats floats) and is taken as zero when the sequence's first
+// row is at position 0.  out [n, heads * v_dim] float32 receives the normalised readout.
+long long shk_mlstm_state_floats(int heads, int dim, int v_dim);
+int shk_mlstm_scan(const float* proj, int ld, int q_off, int k_off, int v_off, int i_off, int f_off,
+                   const float* i_bias, const float* f_bias, float cap, float q_scale, int num_seqs,
+                   int heads, int dim, int v_dim, const int32_t* positions, const int32_t* cu_q,
+                   const int32_t* slots, float* state, long long slot_stride, float* out, void* stream);
+// out[t, h, :] = o[t, h, :] * rsqrt(mean(o[t, h, :]^2) + eps) * weight[h, :] * sigmoid(gate[t, h, :]);
+// o float32 [n, heads * v_dim], gate float32 rows gate_ld apart, out of `dtype`.
+int shk_headnorm_gate(const float* o, const float* gate, int gate_ld, const float* weight, float eps,
+                      void* out, int dtype, int n, int heads, int v_dim, void* stream);
+
+// out = a_pos z^2 + z / 2 where z > 0, a_neg (exp(z) - 1 - z) + z / 2 elsewhere; elementwise.
+int shk_xielu(const void* x, void* out, int dtype, long long numel, float a_pos, float a_neg, void* stream);
+
+// out[i, :] = float(table[ids[i], :]) + float(pair_table[row, :]) with row = (prev * mul_prev +
+// ids[i] * mul_cur) mod buckets, prev the token before token i in its sequence; at position 0,
+// which has none, row = buckets (pair_table has buckets + 1 rows).  For the first token of a
+// step's portion prev is last_token[slots[seq]], where the sequence's step before left its last
+// token; this call leaves the portion's last token there.
+int shk_embed_pairs(const void* table, const void* pair_table, int dtype, const int32_t* ids,
+                    const int32_t* positions, const int32_t* token_seq, const int32_t* cu_q,
+                    const int32_t* slots, int32_t* last_token, float* out, int n, int hidden, int vocab,
+                    int buckets, int mul_prev, int mul_cur, void* stream);
 
 // out[r] = lowest index of the largest value of logits[r, :vocab].  Rows wider
 // than 4096 are searched in chunks; scratch then holds

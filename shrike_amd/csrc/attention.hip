@@ -7,6 +7,9 @@
 // through the block table, with a running maximum and sum, so prompt portions
 // and single decoded tokens take the same path and the same order of
 // operations: a token's result does not depend on how the step was cut.
+// Values may have another size than keys (v_dim); scores may be capped,
+// s <- cap * tanh(s / cap); and the softmax's denominator may hold one more
+// term per head, exp(sinks[head]), that has no key and no value.
 #include "api.h"
 #include "common.h"
 
@@ -18,12 +21,13 @@ constexpr int kMaxHeadDim = 256;
 template <typename T>
 __global__ void __launch_bounds__(kAttnThreads)
     attention_generic_kernel(const T* __restrict__ q, int q_stride, T* __restrict__ out,
-                             int heads, int kv_heads, int head_dim,
+                             int heads, int kv_heads, int head_dim, int v_dim,
                              const int32_t* __restrict__ positions,
                              const int32_t* __restrict__ token_seq,
                              const int32_t* __restrict__ tables, int table_stride,
                              const T* __restrict__ k_pool, const T* __restrict__ v_pool,
-                             int page_size, int num_pages, int window, int chunk, float scale) {
+                             int page_size, int num_pages, int window, int chunk, float scale,
+                             float softcap, const float* __restrict__ sinks) {
   __shared__ float qs[kMaxHeadDim];
   __shared__ float probs[kAttnThreads];
   __shared__ int32_t rows[kAttnThreads];  // key-cache row of each key of the tile, -1 if masked
@@ -41,8 +45,8 @@ __global__ void __launch_bounds__(kAttnThreads)
   __syncthreads();
 
   // PV ownership: thread (g, d) sums keys jj = g, g + groups, ... of a tile for element d.
-  const int groups = kAttnThreads / head_dim;  // >= 1 because head_dim <= 256
-  const int g = threadIdx.x / head_dim, d = threadIdx.x % head_dim;
+  const int groups = kAttnThreads / v_dim;  // >= 1 because v_dim <= 256
+  const int g = threadIdx.x / v_dim, d = threadIdx.x % v_dim;
   const bool pv_active = g < groups;
 
   float m_run = -INFINITY, l_run = 0.f, acc = 0.f;
@@ -64,6 +68,7 @@ __global__ void __launch_bounds__(kAttnThreads)
           kr += static_cast<size_t>(page_size) * slab;
         }
         s = dot * scale;
+        if (softcap > 0.f) s = softcap * tanhf(s / softcap);
       }
     }
     const float m_new = fmaxf(m_run, block_max(s, scratch));
@@ -80,9 +85,9 @@ __global__ void __launch_bounds__(kAttnThreads)
       for (int jj = g; jj < count; jj += groups) {
         const int32_t r = rows[jj];
         if (r < 0) continue;
-        // values are stored [page][kv head][head_dim][page_size]
+        // values are stored [page][kv head][v_dim][page_size]
         const size_t v_at =
-            (static_cast<size_t>(r / page_size) * head_dim + d) * page_size + r % page_size;
+            (static_cast<size_t>(r / page_size) * v_dim + d) * page_size + r % page_size;
         a = fmaf(probs[jj], to_float(v_pool[v_at]), a);
       }
       acc = acc * alpha + a;
@@ -92,11 +97,19 @@ __global__ void __launch_bounds__(kAttnThreads)
 
   partial[threadIdx.x] = pv_active ? acc : 0.f;
   __syncthreads();
-  if (threadIdx.x < head_dim) {
+  // the sink joins the denominator alone: exp(sink) beside the keys' exp(s), nothing in the sum of values
+  float keys_share = 1.f;
+  if (sinks) {
+    const float sink = sinks[head];
+    const float m_all = fmaxf(m_run, sink);
+    keys_share = expf(m_run - m_all);
+    l_run = l_run * keys_share + expf(sink - m_all);
+  }
+  if (threadIdx.x < v_dim) {
     float total = 0.f;
-    for (int gg = 0; gg < groups; ++gg) total += partial[gg * head_dim + threadIdx.x];
-    out[static_cast<size_t>(t) * heads * head_dim + head * head_dim + threadIdx.x] =
-        from_float<T>(total / l_run);
+    for (int gg = 0; gg < groups; ++gg) total += partial[gg * v_dim + threadIdx.x];
+    out[static_cast<size_t>(t) * heads * v_dim + head * v_dim + threadIdx.x] =
+        from_float<T>(total * keys_share / l_run);
   }
 }
 
@@ -108,12 +121,15 @@ extern "C" int shk_attention(const void* q, int q_stride, void* out, int dtype, 
                              int kv_heads, int head_dim, const int32_t* positions,
                              const int32_t* token_seq, const int32_t* tables, int table_stride,
                              int num_seqs, const void* k_pool, const void* v_pool, int page_size,
-                             int num_pages, int window, int chunk, float scale, void* stream) {
+                             int num_pages, int window, int chunk, float scale, int v_dim, float softcap,
+                             const float* sinks, void* stream) {
   SHK_REQUIRE(dtype == kF32 || dtype == kBF16, "attention: unknown dtype %d", dtype);
   SHK_REQUIRE(n >= 0 && heads > 0 && kv_heads > 0 && heads % kv_heads == 0,
               "attention: heads=%d must be a positive multiple of kv_heads=%d", heads, kv_heads);
   SHK_REQUIRE(head_dim > 0 && head_dim <= kMaxHeadDim,
               "attention: head_dim %d is outside 1..%d", head_dim, kMaxHeadDim);
+  SHK_REQUIRE(v_dim > 0 && v_dim <= kAttnThreads, "attention: v_dim %d is outside 1..%d", v_dim, kAttnThreads);
+  SHK_REQUIRE(softcap >= 0.f, "attention: a score cap must be positive (0: none), got %g", softcap);
   SHK_REQUIRE(q_stride >= heads * head_dim, "attention: q_stride %d < heads*head_dim %d", q_stride,
               heads * head_dim);
   SHK_REQUIRE(page_size > 0 && num_pages > 0 && table_stride > 0 && num_seqs > 0,
@@ -129,14 +145,14 @@ extern "C" int shk_attention(const void* q, int q_stride, void* out, int dtype, 
   dim3 grid(heads, n);
   if (dtype == kF32)
     attention_generic_kernel<float><<<grid, kAttnThreads, 0, s>>>(
-        static_cast<const float*>(q), q_stride, static_cast<float*>(out), heads, kv_heads, head_dim,
+        static_cast<const float*>(q), q_stride, static_cast<float*>(out), heads, kv_heads, head_dim, v_dim,
         positions, token_seq, tables, table_stride, static_cast<const float*>(k_pool),
-        static_cast<const float*>(v_pool), page_size, num_pages, window, chunk, scale);
+        static_cast<const float*>(v_pool), page_size, num_pages, window, chunk, scale, softcap, sinks);
   else
     attention_generic_kernel<bf16><<<grid, kAttnThreads, 0, s>>>(
-        static_cast<const bf16*>(q), q_stride, static_cast<bf16*>(out), heads, kv_heads, head_dim,
+        static_cast<const bf16*>(q), q_stride, static_cast<bf16*>(out), heads, kv_heads, head_dim, v_dim,
         positions, token_seq, tables, table_stride, static_cast<const bf16*>(k_pool),
-        static_cast<const bf16*>(v_pool), page_size, num_pages, window, chunk, scale);
+        static_cast<const bf16*>(v_pool), page_size, num_pages, window, chunk, scale, softcap, sinks);
   SHK_LAUNCH_CHECK("attention");
   return 0;
 }

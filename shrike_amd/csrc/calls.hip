@@ -71,6 +71,15 @@ const Launcher kLaunchers[] = {
     SHK_LAUNCHER(shk_attention_decode_bf16),
     SHK_LAUNCHER(shk_attention_prefill_bf16),
     SHK_LAUNCHER(shk_attention_prefill_shared_bf16),
+    SHK_LAUNCHER(shk_qkv_store),
+    SHK_LAUNCHER(shk_latent_prepare),
+    SHK_LAUNCHER(shk_rotate_heads),
+    SHK_LAUNCHER(shk_latent_attention),
+    SHK_LAUNCHER(shk_gemm_batched),
+    SHK_LAUNCHER(shk_mlstm_scan),
+    SHK_LAUNCHER(shk_headnorm_gate),
+    SHK_LAUNCHER(shk_xielu),
+    SHK_LAUNCHER(shk_embed_pairs),
     SHK_LAUNCHER(shk_argmax),
     SHK_LAUNCHER(shk_sample),
 };

@@ -634,3 +634,33 @@ extern "C" int shk_act_mul_rows(const void* a, int a_splits, const void* table, 
   SHK_LAUNCH_CHECK("act_mul_rows");
   return 0;
 }
+
+// ------------------------------------------------------------------ xIELU
+// out = a_pos z^2 + z / 2 for z > 0, a_neg (exp(z) - 1 - z) + z / 2 for z <= 0: an
+// activation with a quadratic positive branch and a negative branch that flattens out;
+// the two factors are the layer's own (learned), given as they are applied.
+namespace shk {
+template <typename T>
+__global__ void xielu_kernel(const T* __restrict__ x, T* __restrict__ out, long long numel, float a_pos, float a_neg) {
+  const long long i = static_cast<long long>(blockIdx.x) * blockDim.x + threadIdx.x;
+  if (i >= numel) return;
+  const float z = to_float(x[i]);
+  const float y = z > 0.f ? fmaf(a_pos * z, z, 0.5f * z) : fmaf(a_neg, expm1f(z) - z, 0.5f * z);
+  out[i] = from_float<T>(y);
+}
+}  // namespace shk
+
+extern "C" int shk_xielu(const void* x, void* out, int dtype, long long numel, float a_pos, float a_neg, void* stream) {
+  SHK_REQUIRE(dtype == kF32 || dtype == kBF16, "xielu: unknown dtype %d", dtype);
+  SHK_REQUIRE(numel >= 0 && numel < (1LL << 31) * 256, "xielu: bad size %lld", numel);
+  if (numel == 0) return 0;
+  SHK_REQUIRE(x && out, "xielu: null pointer");
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  const unsigned grid = static_cast<unsigned>((numel + 255) / 256);
+  if (dtype == kF32)
+    shk::xielu_kernel<float><<<grid, 256, 0, s>>>(static_cast<const float*>(x), static_cast<float*>(out), numel, a_pos, a_neg);
+  else
+    shk::xielu_kernel<shk::bf16><<<grid, 256, 0, s>>>(static_cast<const shk::bf16*>(x), static_cast<shk::bf16*>(out), numel, a_pos, a_neg);
+  SHK_LAUNCH_CHECK("xielu");
+  return 0;
+}

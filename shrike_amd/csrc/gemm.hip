@@ -18,7 +18,12 @@ template <typename TI, typename TO>
 __global__ void __launch_bounds__(256)
     gemm_tiled_kernel(const TI* __restrict__ a, const TI* __restrict__ w,
                       const float* __restrict__ bias, TO* __restrict__ out, int n, int m, int k,
-                      int lda, int ldo, int accumulate) {
+                      int lda, int ldo, int accumulate, long long a_batch, long long w_batch,
+                      long long out_batch) {
+  // blockIdx.z: one of a batch of products of equal shape, operands a fixed step apart
+  a += blockIdx.z * a_batch;
+  w += blockIdx.z * w_batch;
+  out += blockIdx.z * out_batch;
   __shared__ float as[kTK][kTM + 4];
   __shared__ float ws[kTK][kTN + 4];
   const int tx = threadIdx.x % 16, ty = threadIdx.x / 16;
@@ -68,12 +73,13 @@ __global__ void __launch_bounds__(256)
 
 template <typename TI, typename TO>
 static int launch_tiled(const void* a, const void* w, const float* bias, void* out, int n, int m,
-                        int k, int lda, int ldo, int accumulate, hipStream_t s) {
-  dim3 grid((m + kTN - 1) / kTN, (n + kTM - 1) / kTM);
+                        int k, int lda, int ldo, int accumulate, hipStream_t s, int batch = 1,
+                        long long a_batch = 0, long long w_batch = 0, long long out_batch = 0) {
+  dim3 grid((m + kTN - 1) / kTN, (n + kTM - 1) / kTM, batch);
   gemm_tiled_kernel<TI, TO><<<grid, 256, 0, s>>>(static_cast<const TI*>(a),
                                                  static_cast<const TI*>(w), bias,
                                                  static_cast<TO*>(out), n, m, k, lda, ldo,
-                                                 accumulate);
+                                                 accumulate, a_batch, w_batch, out_batch);
   return 0;
 }
 
@@ -103,5 +109,27 @@ extern "C" int shk_gemm(const void* a, const void* w, const float* bias, void* o
   else
     launch_tiled<bf16, bf16>(a, w, bias, out, n, m, k, lda, ldo, accumulate, s);
   SHK_LAUNCH_CHECK("gemm");
+  return 0;
+}
+
+// A batch of products of one shape (one per head, say): product b reads a + b * a_batch
+// (rows lda apart), w + b * w_batch ([m, k] contiguous) and writes out + b * out_batch.
+extern "C" int shk_gemm_batched(const void* a, const void* w, void* out, int n, int m, int k, int lda,
+                                int ldo, int batch, long long a_batch, long long w_batch,
+                                long long out_batch, int dtype, void* stream) {
+  SHK_REQUIRE(dtype == kF32 || dtype == kBF16, "gemm_batched: unknown dtype %d", dtype);
+  SHK_REQUIRE(n >= 0 && m > 0 && k > 0 && batch > 0 && batch <= 65535, "gemm_batched: bad sizes n=%d m=%d k=%d batch=%d",
+              n, m, k, batch);
+  SHK_REQUIRE(lda >= k && ldo >= m, "gemm_batched: row strides lda=%d ldo=%d too small for k=%d m=%d", lda, ldo, k, m);
+  SHK_REQUIRE(a_batch >= 0 && w_batch >= 0 && out_batch >= m, "gemm_batched: outputs of the batch would overlap");
+  if (n == 0) return 0;
+  SHK_REQUIRE(a && w && out, "gemm_batched: null pointer");
+  SHK_REQUIRE((n + kTM - 1) / kTM <= 65535, "gemm_batched: too many rows (%d)", n);
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  if (dtype == kF32)
+    launch_tiled<float, float>(a, w, nullptr, out, n, m, k, lda, ldo, 0, s, batch, a_batch, w_batch, out_batch);
+  else
+    launch_tiled<bf16, bf16>(a, w, nullptr, out, n, m, k, lda, ldo, 0, s, batch, a_batch, w_batch, out_batch);
+  SHK_LAUNCH_CHECK("gemm_batched");
   return 0;
 }

@@ -107,6 +107,10 @@ class ModelRunner:
                 self.layer_caches.append(cache.layer_cache(owner, reader=entry.cache_of is not None))
             else:
                 self.layer_caches.append(None)
+        # state that the embedding keeps per request follows the schedule's positions
+        extra = len(model.spec.schedule)
+        if cache.owns_cache(extra):
+            self.layer_caches.append(cache.layer_cache(extra))
         self._pinned = None
         self._pinned_free = None  # event: the last copy out of the pinned buffer is done
         # Graphs replay fixed kernel arguments: the model's parts say whether

@@ -44,7 +44,16 @@ _SIGNATURES = {
     "shk_mfma_alone": [_P, _P, _I, _I, _P],
     "shk_rope_kv_store": [_P, _I, _I, _I, _I, _I, _I, _P, _P, _P, _P, _I, _P, _P, _I, _I, _I, _P, _I, _P, _I, _I,
                           _P],
-    "shk_attention": [_P, _I, _P, _I, _I, _I, _I, _I, _P, _P, _P, _I, _I, _P, _P, _I, _I, _I, _I, _F, _P],
+    "shk_attention": [_P, _I, _P, _I, _I, _I, _I, _I, _P, _P, _P, _I, _I, _P, _P, _I, _I, _I, _I, _F, _I, _F, _P, _P],
+    "shk_qkv_store": [_P, _I, _I, _I, _I, _I, _I, _F, _I, _F, _P, _P, _P, _I, _P, _P, _I, _I, _I, _P],
+    "shk_latent_prepare": [_P, _I, _I, _I, _I, _I, _P, _P, _F, _P, _P, _P, _P, _I, _P, _P, _I, _I, _I, _P],
+    "shk_rotate_heads": [_P, _I, _I, _I, _P, _I, _I, _I, _I, _I, _I, _I, _P, _P, _P],
+    "shk_latent_attention": [_P, _P, _I, _I, _I, _I, _I, _P, _P, _P, _I, _P, _I, _I, _I, _I, _F, _P],
+    "shk_gemm_batched": [_P, _P, _P, _I, _I, _I, _I, _I, _I, c_longlong, c_longlong, c_longlong, _I, _P],
+    "shk_mlstm_scan": [_P, _I, _I, _I, _I, _I, _I, _P, _P, _F, _F, _I, _I, _I, _I, _P, _P, _P, _P, c_longlong, _P, _P],
+    "shk_headnorm_gate": [_P, _P, _I, _P, _F, _P, _I, _I, _I, _I, _P],
+    "shk_xielu": [_P, _P, _I, c_longlong, _F, _F, _P],
+    "shk_embed_pairs": [_P, _P, _I, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _P],
     "shk_attention_supports_mfma": [_I, _I, _I, _I, _I],
     "shk_attention_decode_bf16": [_P, _I, _P, _I, _I, _I, _I, _P, _P, _I, _P, _P, _I, _I, _I, _F, _P, _I, _I, _P],
     "shk_attention_prefill_bf16": [_P, _I, _P, _I, _I, _I, _I, _P, _P, _P, _P, _P, _I, _P, _P, _I, _I, _I, _F, _P],
@@ -105,6 +114,9 @@ def load():
                 lib._float_slots[launcher_id] = tuple(i for i, t in enumerate(argtypes) if t is c_float)
                 fn = _recorded(fn, launcher_id)
             setattr(lib, name, fn)
+        raw.shk_mlstm_state_floats.argtypes = [_I, _I, _I]
+        raw.shk_mlstm_state_floats.restype = c_longlong
+        lib.shk_mlstm_state_floats = raw.shk_mlstm_state_floats
         raw.shk_sample_scratch_floats.argtypes = [_I, _I]
         raw.shk_sample_scratch_floats.restype = c_longlong
         lib.shk_sample_scratch_floats = raw.shk_sample_scratch_floats

@@ -387,11 +387,13 @@ def key_pool_shape(pages: int, kv_heads: int, page_size: int, head_dim: int) -> 
     return (pages, kv_heads, head_dim // slab, page_size, slab)
 
 
-def _check_pools(who, q, tables, k_pool, v_pool, kv_heads, head_dim, page_size) -> None:
-    """Keys in slabs (key_pool_shape); values transposed [pages, kv_heads, head_dim, page_size]."""
+def _check_pools(who, q, tables, k_pool, v_pool, kv_heads, head_dim, page_size, v_dim=None) -> None:
+    """Keys in slabs (key_pool_shape); values transposed [pages, kv_heads, v_dim, page_size]
+    (v_dim None: values as large as keys)."""
     pages = k_pool.shape[0]
-    if tuple(k_pool.shape) != key_pool_shape(pages, kv_heads, page_size, head_dim):
-        raise KernelError(f"{who}: key pool must be {list(key_pool_shape('pages', kv_heads, page_size, head_dim))}, "
+    key_dim, head_dim = head_dim, (head_dim if v_dim is None else v_dim)
+    if tuple(k_pool.shape) != key_pool_shape(pages, kv_heads, page_size, key_dim):
+        raise KernelError(f"{who}: key pool must be {list(key_pool_shape('pages', kv_heads, page_size, key_dim))}, "
                           f"got {tuple(k_pool.shape)}")
     if tuple(v_pool.shape) != (pages, kv_heads, head_dim, page_size):
         raise KernelError(f"{who}: value pool must be [pages, {kv_heads}, {head_dim}, {page_size}], "
@@ -449,22 +451,216 @@ def rope_kv_store(qkv, heads, kv_heads, head_dim, rot_dim, inv_freq, positions, 
 
 
 def attention(q, out, heads, kv_heads, head_dim, positions, token_seq, tables, k_pool, v_pool,
-              page_size, window, scale, chunk=None) -> None:
-    """q: [n, >= heads*head_dim] rows (a view into qkv is fine); out [n, heads*head_dim]."""
+              page_size, window, scale, chunk=None, v_dim=None, softcap=None, sinks=None) -> None:
+    """q: [n, >= heads*head_dim] rows (a view into qkv is fine); out [n, heads*v_dim].
+    v_dim: size of a value (None: head_dim); softcap: scores become cap * tanh(score / cap);
+    sinks: float32 [heads], one more term exp(sinks[h]) in each head's softmax denominator."""
     _rows(q, "attention q")
     n = q.shape[0]
-    if out.shape != (n, heads * head_dim) or not out.is_contiguous() or out.dtype != q.dtype:
-        raise KernelError("attention: out must be contiguous [n, heads*head_dim] of q's dtype")
-    _check_pools("attention", q, tables, k_pool, v_pool, kv_heads, head_dim, page_size)
+    v_dim = head_dim if v_dim is None else int(v_dim)
+    if out.shape != (n, heads * v_dim) or not out.is_contiguous() or out.dtype != q.dtype:
+        raise KernelError("attention: out must be contiguous [n, heads*v_dim] of q's dtype")
+    if sinks is not None and (sinks.numel() != heads or not sinks.is_contiguous()):
+        raise KernelError(f"attention: sinks must hold one value per head ({heads})")
+    _check_pools("attention", q, tables, k_pool, v_pool, kv_heads, head_dim, page_size, v_dim)
     check(
         load().shk_attention(
             _dev(q, "q"), q.stride(0), _dev(out, "out"), dtype_code(q.dtype), n, heads, kv_heads,
             head_dim, _dev(positions, "positions", torch.int32),
             _dev(token_seq, "token_seq", torch.int32), _dev(tables, "tables", torch.int32),
             tables.shape[1], tables.shape[0], _dev(k_pool, "k_pool"), _dev(v_pool, "v_pool"),
-            page_size, k_pool.shape[0], int(window or 0), int(chunk or 0), float(scale), _stream(),
+            page_size, k_pool.shape[0], int(window or 0), int(chunk or 0), float(scale), v_dim,
+            float(softcap or 0.0), None if sinks is None else _dev(sinks, "sinks", torch.float32), _stream(),
         )
     )
+
+
+def qkv_store(qkv, heads, kv_heads, head_dim, v_dim, positions, token_seq, tables, k_pool, v_pool, page_size,
+              q_temperature=None, v_norm_eps=None, write_kv=True) -> None:
+    """Cache write without rotation for keys of head_dim and values of v_dim: qkv is [n, heads *
+    head_dim + kv_heads * (head_dim + v_dim)].  q_temperature = (coef, every): the queries at
+    position p are multiplied by 1 + coef * ln(floor((p + 1) / every) + 1) in place.
+    v_norm_eps: each head's value is stored divided by sqrt(mean(v^2) + eps)."""
+    n = qkv.shape[0]
+    if not qkv.is_contiguous() or qkv.shape[1] != heads * head_dim + kv_heads * (head_dim + v_dim):
+        raise KernelError("qkv_store: qkv must be contiguous [n, heads*head_dim + kv_heads*(head_dim + v_dim)]")
+    if positions.shape[0] < n or (write_kv and token_seq.shape[0] < n):
+        raise KernelError(f"qkv_store: qkv has {n} rows but positions / token_seq are shorter")
+    num_pages = 0
+    if write_kv:
+        _check_pools("qkv_store", qkv, tables, k_pool, v_pool, kv_heads, head_dim, page_size, v_dim)
+        num_pages = k_pool.shape[0]
+    coef, every = (0.0, 0) if q_temperature is None else (float(q_temperature[0]), int(q_temperature[1]))
+    if q_temperature is not None and every < 1:
+        raise KernelError(f"qkv_store: the query temperature's step must be positive, got {every}")
+    check(load().shk_qkv_store(
+        _dev(qkv, "qkv"), dtype_code(qkv.dtype), n, heads, kv_heads, head_dim, v_dim, coef, every,
+        float(v_norm_eps or 0.0), _dev(positions, "positions", torch.int32),
+        _dev(token_seq, "token_seq", torch.int32) if write_kv else None,
+        _dev(tables, "tables", torch.int32) if write_kv else None, tables.shape[1] if write_kv else 0,
+        _dev(k_pool, "k_pool") if write_kv else None, _dev(v_pool, "v_pool") if write_kv else None,
+        page_size, num_pages, int(bool(write_kv)), _stream()))
+
+
+def latent_prepare(down, q_rank, kv_rank, rot_dim, q_weight, kv_weight, eps, inv_freq, positions, token_seq,
+                   tables, q_latent, pool, page_size, write_kv=True) -> None:
+    """From a token's joint down-projection [q latent | key/value latent | rotated key part]:
+    the normed query latent into q_latent [n, q_rank]; the normed key/value latent and the
+    rotated key part (neighbouring pairs) into the token's row of pool [pages, page_size,
+    kv_rank + rot_dim]."""
+    n = down.shape[0]
+    if not down.is_contiguous() or down.shape[1] != q_rank + kv_rank + rot_dim:
+        raise KernelError("latent_prepare: down must be contiguous [n, q_rank + kv_rank + rot_dim]")
+    if tuple(q_latent.shape) != (n, q_rank) or not q_latent.is_contiguous() or q_latent.dtype != down.dtype:
+        raise KernelError("latent_prepare: q_latent must be contiguous [n, q_rank] of down's dtype")
+    if q_weight.numel() != q_rank or kv_weight.numel() != kv_rank:
+        raise KernelError("latent_prepare: the norms' weights do not fit the latents")
+    if rot_dim and (inv_freq is None or inv_freq.numel() < rot_dim // 2):
+        raise KernelError("latent_prepare: too few rotation rates")
+    if positions.shape[0] < n or (write_kv and token_seq.shape[0] < n):
+        raise KernelError(f"latent_prepare: down has {n} rows but positions / token_seq are shorter")
+    num_pages = 0
+    if write_kv:
+        if (pool.dim() != 3 or tuple(pool.shape[1:]) != (page_size, kv_rank + rot_dim) or not pool.is_contiguous()
+                or pool.dtype != down.dtype or tables.dim() != 2 or not tables.is_contiguous()):
+            raise KernelError(f"latent_prepare: the pool must be contiguous [pages, {page_size}, {kv_rank + rot_dim}] "
+                              "of down's dtype, the tables [sequences, blocks]")
+        num_pages = pool.shape[0]
+    check(load().shk_latent_prepare(
+        _dev(down, "down"), dtype_code(down.dtype), n, q_rank, kv_rank, rot_dim,
+        _dev(q_weight, "q_weight", torch.float32), _dev(kv_weight, "kv_weight", torch.float32), float(eps),
+        None if inv_freq is None else _dev(inv_freq, "inv_freq", torch.float32),
+        _dev(positions, "positions", torch.int32),
+        _dev(token_seq, "token_seq", torch.int32) if write_kv else None,
+        _dev(tables, "tables", torch.int32) if write_kv else None, tables.shape[1] if write_kv else 0,
+        _dev(q_latent, "q_latent"), _dev(pool, "pool") if write_kv else None, page_size, num_pages,
+        int(bool(write_kv)), _stream()))
+
+
+def rotate_heads(src, src_head, src_off, dst, dst_head, dst_off, heads, rot_dim, inv_freq, positions) -> None:
+    """dst[t, h*dst_head + dst_off + e] = rotation of src[t, h*src_head + src_off + e] for e < rot_dim:
+    neighbouring pairs (2i, 2i + 1) turned by positions[t] * inv_freq[i]."""
+    _rows(src, "rotate_heads src")
+    _rows(dst, "rotate_heads dst")
+    n = src.shape[0]
+    if dst.shape[0] != n or src.dtype != dst.dtype or positions.shape[0] < n:
+        raise KernelError("rotate_heads: src, dst and positions differ in rows or dtype")
+    if src.shape[1] < heads * src_head or dst.shape[1] < heads * dst_head:
+        raise KernelError("rotate_heads: the rows are shorter than heads * head size")
+    if rot_dim and (inv_freq is None or inv_freq.numel() < rot_dim // 2):
+        raise KernelError("rotate_heads: too few rotation rates")
+    check(load().shk_rotate_heads(
+        _dev(src, "src"), src.stride(0), src_head, src_off, _dev(dst, "dst"), dst.stride(0), dst_head, dst_off,
+        dtype_code(src.dtype), n, heads, rot_dim,
+        None if inv_freq is None else _dev(inv_freq, "inv_freq", torch.float32),
+        _dev(positions, "positions", torch.int32), _stream()))
+
+
+def latent_attention(q, out, heads, key_dim, v_dim, positions, token_seq, tables, pool, page_size, window,
+                     scale, chunk=None) -> None:
+    """q [n, heads * key_dim], out [n, heads * v_dim]; pool [pages, page_size, key_dim]: a row is a
+    key, its first v_dim elements the value; every head reads the same rows."""
+    n = q.shape[0]
+    if tuple(q.shape) != (n, heads * key_dim) or not q.is_contiguous():
+        raise KernelError("latent_attention: q must be contiguous [n, heads * key_dim]")
+    if tuple(out.shape) != (n, heads * v_dim) or not out.is_contiguous() or out.dtype != q.dtype:
+        raise KernelError("latent_attention: out must be contiguous [n, heads * v_dim] of q's dtype")
+    if (pool.dim() != 3 or tuple(pool.shape[1:]) != (page_size, key_dim) or not pool.is_contiguous()
+            or pool.dtype != q.dtype or tables.dim() != 2 or not tables.is_contiguous()):
+        raise KernelError(f"latent_attention: the pool must be contiguous [pages, {page_size}, {key_dim}] of q's dtype")
+    if positions.shape[0] < n or token_seq.shape[0] < n:
+        raise KernelError("latent_attention: positions / token_seq are shorter than q")
+    check(load().shk_latent_attention(
+        _dev(q, "q"), _dev(out, "out"), dtype_code(q.dtype), n, heads, key_dim, v_dim,
+        _dev(positions, "positions", torch.int32), _dev(token_seq, "token_seq", torch.int32),
+        _dev(tables, "tables", torch.int32), tables.shape[1], _dev(pool, "pool"), page_size, pool.shape[0],
+        int(window or 0), int(chunk or 0), float(scale), _stream()))
+
+
+def gemm_batched(a, w, out, batch: int, a_step: int, out_step: int) -> None:
+    """out[:, b*out_step : b*out_step + m] = a[:, b*a_step : b*a_step + k] @ w[b].T for b < batch;
+    w [batch, m, k] contiguous; a and out 2-d with unit inner stride; all of one dtype."""
+    _rows(a, "gemm_batched a")
+    _rows(out, "gemm_batched out")
+    n = a.shape[0]
+    if w.dim() != 3 or w.shape[0] != batch or not w.is_contiguous() or w.dtype != a.dtype or out.dtype != a.dtype:
+        raise KernelError("gemm_batched: w must be contiguous [batch, m, k] of a's dtype, as out is")
+    m, k = w.shape[1], w.shape[2]
+    if out.shape[0] != n or (batch - 1) * a_step + k > a.shape[1] or (batch - 1) * out_step + m > out.shape[1] \
+            or out_step < m or a_step < 0:
+        raise KernelError("gemm_batched: the batch's slices do not fit a or out")
+    check(load().shk_gemm_batched(_dev(a, "a"), _dev(w, "w"), _dev(out, "out"), n, m, k, a.stride(0), out.stride(0),
+                                  batch, a_step, m * k, out_step, dtype_code(a.dtype), _stream()))
+
+
+def mlstm_state_floats(heads: int, dim: int, v_dim: int) -> int:
+    """float32 values of one request's state in one mLSTM layer (mlstm_scan's own layout)."""
+    return int(load().shk_mlstm_state_floats(heads, dim, v_dim))
+
+
+def mlstm_scan(proj, q_off, k_off, v_off, i_off, f_off, i_bias, f_bias, cap, q_scale, num_seqs, heads, dim, v_dim,
+               positions, cu_q, slots, state, out) -> None:
+    """The mLSTM recurrence over the step's tokens.  proj float32 [n, ld] holds the projections
+    at the given column offsets; state float32 [slots(+1), state floats]; out float32
+    [n, heads * v_dim]."""
+    _rows(proj, "mlstm_scan proj")
+    n = proj.shape[0]
+    if proj.dtype != torch.float32 or out.dtype != torch.float32 or tuple(out.shape) != (n, heads * v_dim) \
+            or not out.is_contiguous():
+        raise KernelError("mlstm_scan: proj and out must be float32, out contiguous [n, heads * v_dim]")
+    if state.dim() != 2 or state.dtype != torch.float32 or state.stride(1) != 1:
+        raise KernelError("mlstm_scan: state must be float32 [slots, floats]")
+    if cu_q.shape[0] < num_seqs + 1 or slots.shape[0] < num_seqs:
+        raise KernelError("mlstm_scan: cu_q / slots are shorter than the step's sequences")
+    if i_bias.numel() != heads or f_bias.numel() != heads:
+        raise KernelError("mlstm_scan: one gate bias per head")
+    check(load().shk_mlstm_scan(
+        _dev(proj, "proj"), proj.stride(0), q_off, k_off, v_off, i_off, f_off,
+        _dev(i_bias, "i_bias", torch.float32), _dev(f_bias, "f_bias", torch.float32), float(cap), float(q_scale),
+        num_seqs, heads, dim, v_dim, _dev(positions, "positions", torch.int32), _dev(cu_q, "cu_q", torch.int32),
+        _dev(slots, "slots", torch.int32), _dev(state, "state"), state.stride(0), _dev(out, "out"), _stream()))
+
+
+def headnorm_gate(o, gate, weight, eps, out, heads, v_dim) -> None:
+    """out[t, h] = o[t, h] / rms(o[t, h]) * weight[h] * sigmoid(gate[t, h]); o float32 [n, heads * v_dim],
+    gate float32 rows (a view with a row stride is fine), out of the compute dtype."""
+    _rows(gate, "headnorm_gate gate")
+    n = o.shape[0]
+    if o.dtype != torch.float32 or gate.dtype != torch.float32 or not o.is_contiguous() or not out.is_contiguous() \
+            or tuple(o.shape) != (n, heads * v_dim) or tuple(out.shape) != (n, heads * v_dim) \
+            or gate.shape[0] != n or gate.shape[1] < heads * v_dim or weight.numel() != heads * v_dim:
+        raise KernelError("headnorm_gate: o, gate float32 [n, heads * v_dim], out alike in the compute dtype")
+    check(load().shk_headnorm_gate(_dev(o, "o"), _dev(gate, "gate"), gate.stride(0),
+                                   _dev(weight, "weight", torch.float32), float(eps), _dev(out, "out"),
+                                   dtype_code(out.dtype), n, heads, v_dim, _stream()))
+
+
+def xielu(x, out, a_pos: float, a_neg: float) -> None:
+    """out = a_pos x^2 + x / 2 where x > 0, a_neg (exp(x) - 1 - x) + x / 2 elsewhere."""
+    if x.shape != out.shape or x.dtype != out.dtype or not x.is_contiguous() or not out.is_contiguous():
+        raise KernelError("xielu: x and out must be contiguous and alike")
+    check(load().shk_xielu(_dev(x, "x"), _dev(out, "out"), dtype_code(x.dtype), x.numel(), float(a_pos),
+                           float(a_neg), _stream()))
+
+
+def embed_pairs(table, pair_table, ids, positions, token_seq, cu_q, slots, last_token, out, buckets, mul_prev,
+                mul_cur) -> None:
+    """out[i] = table[ids[i]] + pair_table[hash(previous token, ids[i])] in float32; the token before a
+    step's first one comes from last_token[slots[seq]] (int32 [slots(+1)]), which receives the
+    step's last one."""
+    n, hidden = out.shape
+    if not (table.is_contiguous() and pair_table.is_contiguous() and out.is_contiguous()) \
+            or table.shape[1] != hidden or tuple(pair_table.shape) != (buckets + 1, hidden) \
+            or pair_table.dtype != table.dtype:
+        raise KernelError("embed_pairs: table [vocab, hidden], pair_table [buckets + 1, hidden], out [n, hidden]")
+    if last_token.dtype != torch.int32 or not last_token.is_contiguous():
+        raise KernelError("embed_pairs: last_token must be contiguous int32")
+    check(load().shk_embed_pairs(
+        _dev(table, "table"), _dev(pair_table, "pair_table"), dtype_code(table.dtype),
+        _dev(ids, "ids", torch.int32), _dev(positions, "positions", torch.int32),
+        _dev(token_seq, "token_seq", torch.int32), _dev(cu_q, "cu_q", torch.int32),
+        _dev(slots, "slots", torch.int32), _dev(last_token, "last_token"), _dev(out, "out", torch.float32),
+        n, hidden, table.shape[0], int(buckets), int(mul_prev), int(mul_cur), _stream()))
 
 
 def attention_supports_mfma(heads, kv_heads, head_dim, page_size, q_stride) -> bool:

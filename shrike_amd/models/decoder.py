@@ -23,6 +23,11 @@ class DecoderModel:
         self.head = build_part("head", spec.head, h, spec.head_name)
         if spec.tie_word_embeddings:
             self.head.tie(self.embedding)
+        # an embedding that depends on the token before keeps it per request, as mixers keep state
+        spec_of = getattr(self.embedding, "cache_spec", None)
+        self.embedding_state = spec_of() if spec_of is not None else None
+        if self.embedding_state is not None and not isinstance(self.embedding_state, StateSpec):
+            raise TypeError("an embedding's cache need must be a StateSpec")
         # some run adds the embedding's output to the stream again: it is kept
         self._keep_embedding = any(e.add_embedding for e in spec.schedule)
         self.stream_vectors: dict = {}
@@ -58,6 +63,8 @@ class DecoderModel:
             mixer = block.mixer
             if isinstance(mixer.cache_spec(), StateSpec) and not mixer.state_graph_safe:
                 return False
+        if self.embedding_state is not None and not getattr(self.embedding, "state_graph_safe", False):
+            return False
         return True
 
     def launches_follow_shape(self) -> bool:
@@ -68,11 +75,15 @@ class DecoderModel:
 
     def cache_specs(self) -> list:
         """Cache need of every schedule position (None for a position that
-        reads another position's cache or whose mixer keeps nothing)."""
+        reads another position's cache or whose mixer keeps nothing), and after
+        them, where the embedding keeps state per request, one more entry for it
+        (position len(schedule))."""
         out = []
         for entry in self.spec.schedule:
             mixer = self.blocks[entry.block].mixer
             out.append(None if entry.cache_of is not None else mixer.cache_spec())
+        if self.embedding_state is not None:
+            out.append(self.embedding_state)
         return out
 
     def load(self, tensors: dict[str, torch.Tensor], runtime) -> None:
@@ -97,7 +108,10 @@ class DecoderModel:
     def forward(self, ctx, caches) -> torch.Tensor:
         """Logits float32 [R, vocab] at ctx.out_rows.  `caches[i]` is the
         LayerCache of schedule position i."""
-        hidden = HiddenState(self.embedding.forward(ctx))
+        if self.embedding_state is not None:
+            hidden = HiddenState(self.embedding.forward(ctx, cache=caches[len(self.spec.schedule)]))
+        else:
+            hidden = HiddenState(self.embedding.forward(ctx))
         embedded = self.embedding.forward(ctx, into="embedded") if self._keep_embedding else None
         for pos, entry in enumerate(self.spec.schedule):
             if entry.add_embedding or entry.add_vector is not None:

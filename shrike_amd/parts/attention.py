@@ -31,18 +31,19 @@ def compute_units() -> int:
 
 
 def kv_cache_spec(num_kv_heads: int, head_dim: int, window: int | None = None,
-                  chunk: int | None = None) -> PagedSpec:
+                  chunk: int | None = None, value_dim: int | None = None) -> PagedSpec:
     """The cache of grouped-query attention, laid out for this file's kernels: per
     page and key/value head the keys in slabs of 32 elements, [head_dim / 32,
     page_size, 32] (a wavefront's operand load for the matrix instruction then
     touches whole cache lines: 64 bytes from each of four consecutive keys; one
     slab of head_dim elements where head_dim is no multiple of 32), and the values
     transposed, [head_dim, page_size] (the keys of a page side by side for every
-    element, which is the operand layout of V^T)."""
+    element, which is the operand layout of V^T).  `value_dim`: the size of a value
+    where it is not the keys' size."""
     slab = ops.key_slab(head_dim)
     return PagedSpec(
         tensors=(PageTensor("k", (num_kv_heads, head_dim // slab, PAGE, slab)),
-                 PageTensor("v", (num_kv_heads, head_dim, PAGE))),
+                 PageTensor("v", (num_kv_heads, head_dim if value_dim is None else value_dim, PAGE))),
         window=window,
         chunk=chunk,
     )
@@ -152,14 +153,31 @@ class PagedAttention(Mixer):
             build_part("position", spec.position, width, name) if spec.position is not None else None
         )
 
+    @property
+    def value_dim(self) -> int:
+        s = self.spec
+        return s.head_dim if getattr(s, "value_dim", None) is None else int(s.value_dim)
+
+    @property
+    def plain_store(self) -> bool:
+        """Whether the step goes through the cache-write kernel without rotation that
+        takes values of another size than keys, the queries' temperature and the
+        values' unit norm, and through the general attention kernel."""
+        s = self.spec
+        return bool(self.value_dim != s.head_dim or getattr(s, "query_temperature", None)
+                    or getattr(s, "value_norm_eps", None) or getattr(s, "softcap", None)
+                    or getattr(s, "sinks", False))
+
     def params(self):
         s, h = self.spec, self.width
         q, kv = s.num_heads * s.head_dim, s.num_kv_heads * s.head_dim
         t = self._tensor
         out = [ParamSpec(t("q"), (q, h)), ParamSpec(t("k"), (kv, h))]
         if not s.values_from_keys:
-            out.append(ParamSpec(t("v"), (kv, h)))
-        out.append(ParamSpec(t("o"), (h, q)))
+            out.append(ParamSpec(t("v"), (s.num_kv_heads * self.value_dim, h)))
+        out.append(ParamSpec(t("o"), (h, s.num_heads * self.value_dim)))
+        if getattr(s, "sinks", False):
+            out.append(ParamSpec(t("sink"), (s.num_heads,), init="bias", keep_float32=True))
         if s.qkv_bias:
             out += [ParamSpec(t(f"{r}_bias"), (q if r == "q" else kv,), init="bias", keep_float32=True)
                     for r in ("q", "k") + (() if s.values_from_keys else ("v",))]
@@ -169,17 +187,30 @@ class PagedAttention(Mixer):
 
     _DEFAULT_NAMES = {"q": "q_proj.weight", "k": "k_proj.weight", "v": "v_proj.weight", "o": "o_proj.weight",
                       "q_bias": "q_proj.bias", "k_bias": "k_proj.bias", "v_bias": "v_proj.bias",
-                      "o_bias": "o_proj.bias"}
+                      "o_bias": "o_proj.bias", "sink": "sinks"}
 
     def _tensor(self, role: str) -> str:
         return self.tensor_name(role, self._DEFAULT_NAMES[role])
 
     def cache_spec(self):
         s = self.spec
-        return kv_cache_spec(s.num_kv_heads, s.head_dim, s.window, s.chunk)
+        return kv_cache_spec(s.num_kv_heads, s.head_dim, s.window, s.chunk,
+                             None if self.value_dim == s.head_dim else self.value_dim)
 
     def check(self, runtime):
         s = self.spec
+        if self.plain_store:
+            if self.position is not None or s.values_from_keys or s.qkv_bias:
+                raise ValueError(f"{self.name}: values of another size than keys, a query temperature, normed "
+                                 "values, capped scores and sinks are built for attention without rotation, "
+                                 "without biases on q, k, v and with values of their own")
+            if not 1 <= self.value_dim <= 256:
+                raise ValueError(f"{self.name}: value_dim {self.value_dim} is outside 1..256")
+            qt = getattr(s, "query_temperature", None)
+            if qt is not None and (len(qt) != 2 or int(qt[1]) < 1):
+                raise ValueError(f"{self.name}: query_temperature must be (coef, every) with every >= 1, got {qt}")
+            if getattr(s, "softcap", None) is not None and not s.softcap > 0:
+                raise ValueError(f"{self.name}: softcap must be positive, got {s.softcap}")
         if s.num_heads % s.num_kv_heads:
             raise ValueError(
                 f"{self.name}: {s.num_heads} query heads are not a multiple of "
@@ -203,6 +234,7 @@ class PagedAttention(Mixer):
         self.b_qkv = torch.cat([tensors[t(f"{r}_bias")] for r in roles]).contiguous() if s.qkv_bias else None
         self.w_o = runtime.weight(tensors[t("o")])
         self.b_o = tensors[t("o_bias")] if s.out_bias else None
+        self.sinks = tensors[t("sink")].contiguous() if getattr(s, "sinks", False) else None
         if self.position is not None:
             self.position.load(tensors, runtime)
         self.linear = runtime.linear
@@ -214,7 +246,7 @@ class PagedAttention(Mixer):
     @property
     def plan_key(self):
         s = self.spec
-        return ("paged_attention", s.num_heads, s.num_kv_heads, s.head_dim, s.window, s.chunk)
+        return ("paged_attention", s.num_heads, s.num_kv_heads, s.head_dim, s.window, s.chunk, self.plain_store)
 
     def prepare(self, shape) -> None:
         """Decides once per step and head geometry how attention is launched:
@@ -226,7 +258,7 @@ class PagedAttention(Mixer):
         s = self.spec
         h, hkv, d = s.num_heads, s.num_kv_heads, s.head_dim
         plan = shape.notes[key] = AttentionPlan()
-        plan.mfma = self.dtype == torch.bfloat16 and ops.attention_supports_mfma(
+        plan.mfma = self.dtype == torch.bfloat16 and not self.plain_store and ops.attention_supports_mfma(
             h, hkv, d, shape.page_size, self._qkv_width())
         # the most keys that any query reads, where the mask bounds them
         reach = min(x for x in (s.window, s.chunk, 1 << 40) if x)
@@ -285,7 +317,8 @@ class PagedAttention(Mixer):
         q = qkv[:, : h * d]
         if not plan.mfma:
             ops.attention(q, out, h, hkv, d, ctx.positions, ctx.token_seq, tables, cache.pools["k"],
-                          cache.pools["v"], cache.page_size, s.window, s.scale, chunk=s.chunk)
+                          cache.pools["v"], cache.page_size, s.window, s.scale, chunk=s.chunk,
+                          v_dim=self.value_dim, softcap=getattr(s, "softcap", None), sinks=self.sinks)
             return
         if ctx.num_decode:
             partial = ctx.buffer("attn_partial", (ctx.num_decode * h * plan.nsplit * (d + 2),),
@@ -313,12 +346,25 @@ class PagedAttention(Mixer):
 
     def _qkv_width(self) -> int:
         s = self.spec
-        return (s.num_heads + (1 if s.values_from_keys else 2) * s.num_kv_heads) * s.head_dim
+        if s.values_from_keys:
+            return (s.num_heads + s.num_kv_heads) * s.head_dim
+        return (s.num_heads + s.num_kv_heads) * s.head_dim + s.num_kv_heads * self.value_dim
 
     def forward(self, ctx, x: torch.Tensor, cache) -> torch.Tensor:
         s = self.spec
         n = x.shape[0]
         qkv_width = self._qkv_width()
+        if self.plain_store:
+            qkv = ctx.buffer("attn_qkv", (n, qkv_width), ctx.dtype)
+            self.linear(x, self.w_qkv, qkv)
+            tables = ctx.block_tables[cache.group]
+            ops.qkv_store(qkv, s.num_heads, s.num_kv_heads, s.head_dim, self.value_dim, ctx.positions,
+                          ctx.token_seq, tables, cache.pools["k"], cache.pools["v"], cache.page_size,
+                          q_temperature=getattr(s, "query_temperature", None),
+                          v_norm_eps=getattr(s, "value_norm_eps", None), write_kv=cache.owned)
+            attn = ctx.buffer("attn_out", (n, s.num_heads * self.value_dim), ctx.dtype)
+            self.attend(ctx, qkv, attn, tables, cache)
+            return self.linear_deferred(ctx, "attn_proj", attn, self.w_o, bias=self.b_o)
         table = self.position.rotary_table() if self.position is not None else None
         fused_position = self.position is None or table is not None
         split_sum = None

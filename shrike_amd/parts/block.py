@@ -13,9 +13,12 @@ class PreNormResidualBlock(Block):
         super().__init__(spec, width, name)
         self.mixer_norm = build_part("norm", spec.mixer_norm, width, f"{name}.{spec.mixer_norm_name}")
         self.mixer = build_part("mixer", spec.mixer, width, f"{name}.{spec.mixer_name}")
-        self.ffn_norm = build_part("norm", spec.ffn_norm, width, f"{name}.{spec.ffn_norm_name}")
-        self.ffn = build_part("ffn", spec.ffn, width, f"{name}.{spec.ffn_name}")
-        self.parts = (self.mixer_norm, self.mixer, self.ffn_norm, self.ffn)
+        # a layer without a feed-forward has no second norm either
+        self.ffn_norm = self.ffn = None
+        if spec.ffn is not None:
+            self.ffn_norm = build_part("norm", spec.ffn_norm, width, f"{name}.{spec.ffn_norm_name}")
+            self.ffn = build_part("ffn", spec.ffn, width, f"{name}.{spec.ffn_name}")
+        self.parts = tuple(p for p in (self.mixer_norm, self.mixer, self.ffn_norm, self.ffn) if p is not None)
 
     def params(self):
         return [p for part in self.parts for p in part.params()]
@@ -39,6 +42,8 @@ class PreNormResidualBlock(Block):
     def forward(self, ctx, hidden: HiddenState, cache) -> None:
         x = self.mixer_norm.forward(ctx, hidden)
         hidden.pending = self.mixer.forward(ctx, x, cache)
+        if self.ffn is None:
+            return
         x = self.ffn_norm.forward(ctx, hidden)
         hidden.pending = self.ffn.forward(ctx, x)
 

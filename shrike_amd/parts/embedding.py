@@ -5,7 +5,7 @@ from __future__ import annotations
 import torch
 
 from ..kernels import ops
-from .base import Embedding, ParamSpec, register_embedding
+from .base import Embedding, ParamSpec, StateSpec, register_embedding
 
 
 class TokenEmbedding(Embedding):
@@ -30,3 +30,47 @@ class TokenEmbedding(Embedding):
 
 
 register_embedding("token_lookup", TokenEmbedding)
+
+
+class PairHashEmbedding(Embedding):
+    """x[n] = table[token] + pairs[(previous token * mul_prev + token * mul_cur) mod buckets],
+    summed in float32; the first token of a sequence takes the pair table's last row.  The
+    token before a step's first token is part of the request's state: it lives in the
+    request's state slot on the device (one int32), where the kernel reads it and leaves
+    the step's last token, so steps replayed from graphs or launched ahead of the host find
+    it without the host's help."""
+
+    launches_follow_shape = True
+    state_graph_safe = True
+
+    def params(self):
+        s = self.spec
+        return [ParamSpec(self.tensor_name("weight"), (s.vocab_size, self.width), init="embedding"),
+                ParamSpec(s.pair_name, (s.buckets + 1, self.width), init="embedding")]
+
+    def cache_spec(self):
+        return StateSpec((1,), "int32")
+
+    def check(self, runtime):
+        s = self.spec
+        if s.buckets < 1:
+            raise ValueError(f"{self.name}: buckets must be positive, got {s.buckets}")
+        if max(abs(int(s.mul_prev)), abs(int(s.mul_cur))) >= 1 << 31:
+            raise ValueError(f"{self.name}: the hash's multipliers must fit 32 bits")
+
+    def load(self, tensors, runtime):
+        self.table = tensors[self.tensor_name("weight")]
+        self.pairs = tensors[self.spec.pair_name]
+
+    def forward(self, ctx, into: str = "resid", cache=None) -> torch.Tensor:
+        if cache is None or into != "resid":
+            raise RuntimeError(f"{self.name}: the pair embedding runs once a step, with its state")
+        s = self.spec
+        resid = ctx.buffer(into, (ctx.num_tokens, self.width), torch.float32)
+        state = cache.state_padded if cache.state_padded is not None else cache.state
+        ops.embed_pairs(self.table, self.pairs, ctx.token_ids, ctx.positions, ctx.token_seq, ctx.cu_q,
+                        ctx.state_slots, state.view(-1), resid, s.buckets, s.mul_prev, s.mul_cur)
+        return resid
+
+
+register_embedding("token_pair_hash", PairHashEmbedding)

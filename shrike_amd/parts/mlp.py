@@ -47,3 +47,47 @@ class SwiGLU(FeedForward):
 
 
 register_ffn("swiglu", SwiGLU)
+
+
+class DenseFFN(FeedForward):
+    """down(act(up(x))) without biases.  The xIELU activation has two learned numbers
+    per layer (a tensor of two elements, p and q): softplus(p) scales the quadratic
+    branch for z > 0, 1/2 + softplus(q) the flattening branch for z <= 0; both are
+    formed once, in float32, when the weights are loaded."""
+
+    launches_follow_shape = True
+
+    def params(self):
+        inter, h = self.spec.intermediate_size, self.width
+        return [
+            ParamSpec(self.tensor_name("up", "up_proj.weight"), (inter, h)),
+            ParamSpec(self.tensor_name("down", "down_proj.weight"), (h, inter)),
+            ParamSpec(self.tensor_name("act", "act"), (2,), init="bias", keep_float32=True),
+        ]
+
+    def check(self, runtime):
+        if self.spec.activation != "xielu":
+            raise ValueError(f"{self.name}: the dense feed-forward's activation must be 'xielu', "
+                             f"got {self.spec.activation!r}")
+
+    def load(self, tensors, runtime):
+        self.inter = int(self.spec.intermediate_size)
+        self.w_up = runtime.weight(tensors[self.tensor_name("up", "up_proj.weight")])
+        self.w_down = runtime.weight(tensors[self.tensor_name("down", "down_proj.weight")])
+        p, q = torch.nn.functional.softplus(tensors[self.tensor_name("act", "act")].to(torch.float32)).tolist()
+        self.a_pos, self.a_neg = float(p), 0.5 + float(q)
+        self.linear = runtime.linear
+        self.linear_deferred = runtime.linear_deferred
+
+    def forward(self, ctx, x: torch.Tensor) -> torch.Tensor:
+        from ..kernels import ops
+
+        n = x.shape[0]
+        up = ctx.buffer("ffn_up", (n, self.inter), ctx.dtype)
+        self.linear(x, self.w_up, up)
+        act = ctx.buffer("ffn_act", (n, self.inter), ctx.dtype)
+        ops.xielu(up, act, self.a_pos, self.a_neg)
+        return self.linear_deferred(ctx, "ffn_out", act, self.w_down)
+
+
+register_ffn("dense_act", DenseFFN)

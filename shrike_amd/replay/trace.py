@@ -37,6 +37,8 @@ def main(argv=None) -> int:
     ap.add_argument("--max-tokens", type=int, required=True,
                     help="most tokens live requests hold at any time (each rounded up to 64)")
     ap.add_argument("--block-size", type=int, default=16, help="tokens per cache page")
+    ap.add_argument("--max-requests", type=int, default=4,
+                    help="state slots: the most requests that are live at any time")
     ap.add_argument("--no-graphs", action="store_true", help="launch every step kernel by kernel")
     ap.add_argument("--poison", action="store_true",
                     help="fill pages that no request holds with NaN (at start and when given back)")
@@ -62,7 +64,7 @@ def main(argv=None) -> int:
     model, runtime, _cfg = load_model(args.model, args.dtype)
     page = args.block_size
     num_pages = max(1, -(-args.max_tokens // page))
-    cache = CacheManager(model.cache_specs(), page, num_pages, max_slots=64,
+    cache = CacheManager(model.cache_specs(), page, num_pages, max_slots=args.max_requests,
                          enable_prefix_caching=False)
     cache.allocate(runtime.dtype, runtime.device)
     runner = ModelRunner(model, cache, runtime, graphs=not args.no_graphs)
