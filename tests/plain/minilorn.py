@@ -91,15 +91,17 @@ def attention_mixer(h, positions, w, prefix: str, m: dict, eps: float):
     return out.reshape(n, H * V) @ w[prefix + ".o"].T
 
 
-def rotate_interleaved(x, positions, base: float, dims: int):
-    """x [..., tokens, dim] with tokens on the second-to-last axis... here [tokens, heads, dim].
-    Elements 2i and 2i+1 (i < dims/2) turn by positions * base**(-2i/dims)."""
+def rotate_interleaved(x, positions, base: float, dims: int, angle_dtype=None):
+    """x [tokens, heads, dim].  Elements 2i and 2i+1 (i < dims/2) turn by positions *
+    base**(-2i/dims).  The design forms positions and angles in 32-bit: with
+    angle_dtype=torch.float32 the rates are rounded to it and the product is formed in it
+    (thousands of radians are then known to about 1e-4); otherwise in float64."""
     out = x.clone()
     if dims == 0:
         return out
     i = torch.arange(dims // 2, dtype=torch.float64)
-    rate = base ** (-2.0 * i / dims)
-    angle = (positions.to(torch.float64)[:, None] * rate[None, :]).to(x.dtype)
+    rate = (base ** (-2.0 * i / dims)).to(angle_dtype or torch.float64)
+    angle = (positions.to(rate.dtype)[:, None] * rate[None, :]).to(torch.float64).to(x.dtype)
     c, s = torch.cos(angle)[:, None, :], torch.sin(angle)[:, None, :]
     u, v = x[..., 0:dims:2], x[..., 1:dims:2]
     out[..., 0:dims:2] = u * c - v * s
@@ -208,3 +210,33 @@ def forward(cfg: dict, w: dict, tokens, return_layers: bool = False):
         layers.append(x)
     logits = weighted_norm(x, w["final.norm"], eps) @ w["head"].T
     return (logits, torch.stack(layers)) if return_layers else logits
+
+
+class PlainMinilorn:
+    """A model folder read once; `logits(ids)`, the stream after every layer, and greedy
+    generation over it, in float64 unless told otherwise."""
+
+    def __init__(self, model_dir, dtype=torch.float64):
+        import json
+        from pathlib import Path
+
+        from safetensors.torch import load_file
+
+        self.cfg = json.loads((Path(model_dir) / "config.json").read_text())
+        raw = load_file(str(Path(model_dir) / "model.safetensors"))
+        self.weights = {k: (v.to(dtype) if v.is_floating_point() else v) for k, v in raw.items()}
+
+    def logits(self, token_ids, rows=None) -> torch.Tensor:
+        out = forward(self.cfg, self.weights, list(token_ids))
+        return out if rows is None else out[torch.tensor(list(rows), dtype=torch.long)]
+
+    def layers(self, token_ids) -> torch.Tensor:
+        return forward(self.cfg, self.weights, list(token_ids), return_layers=True)[1]
+
+    def greedy(self, prompt, max_new_tokens: int) -> list[int]:
+        seq, out = list(prompt), []
+        for _ in range(max_new_tokens):
+            tok = int(torch.argmax(self.logits(seq)[-1]))
+            out.append(tok)
+            seq.append(tok)
+        return out
