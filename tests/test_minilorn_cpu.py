@@ -8,7 +8,7 @@ import pytest
 import torch
 
 import shrike_amd.models  # noqa: F401  (registers the architectures)
-from shrike_amd.config.registry import ConfigError, get_architecture
+from shrike_amd.config import registry  # (names through the module: another test reloads it)
 from shrike_amd.models import DecoderModel
 from shrike_amd.parts import PagedSpec, StateSpec
 
@@ -19,7 +19,7 @@ D = torch.float64
 
 
 def test_config_reads_back_and_picks_the_parts():
-    arch = get_architecture("Minilorn")
+    arch = registry.get_architecture("Minilorn")
     for name, raw in CONFIGS.items():
         cfg = arch.config_cls.from_dict(raw)
         again = arch.config_cls.from_dict(cfg.to_dict())
@@ -60,8 +60,8 @@ def test_config_reads_back_and_picks_the_parts():
 def test_config_errors_name_the_key(change, message):
     raw = copy.deepcopy(CONFIGS["A"])
     change(raw)
-    with pytest.raises(ConfigError, match=message):
-        get_architecture("Minilorn").config_cls.from_dict(raw)
+    with pytest.raises(registry.ConfigError, match=message):
+        registry.get_architecture("Minilorn").config_cls.from_dict(raw)
 
 
 def test_pair_rows_by_hand():
@@ -202,7 +202,7 @@ def test_matrix_memory_carries_its_state_and_equals_the_unstabilised_sum():
 def test_the_whole_model_is_causal_and_its_first_token_stands_alone(name):
     from shrike_amd.weights.random_init import random_tensor
 
-    arch = get_architecture("Minilorn")
+    arch = registry.get_architecture("Minilorn")
     spec = arch.build_spec(arch.config_cls.from_dict(CONFIGS[name]))
     w = {p.name: random_tensor(p, 1, torch.float32, mode="unit").double() for p in DecoderModel(spec).params()}
     vocab = CONFIGS[name]["vocab"]
