@@ -67,6 +67,8 @@ def matmul_params(cfg) -> tuple[int, int]:
 
 
 def kv_bytes_per_token(cfg) -> int:
+    if getattr(cfg, "kv_elements_per_token", None) is not None:  # a design whose layers cache other things
+        return cfg.kv_elements_per_token * 2
     return cfg.num_hidden_layers * 2 * cfg.num_key_value_heads * cfg.head_dim * 2
 
 
@@ -319,7 +321,9 @@ def kernel_breakdown(engine, steps: int = 3, before_step=None) -> dict:
 
     names = ["embed", "add_rmsnorm", "act_mul", "gemm", "gemm_tiled_weight", "rope_kv_store", "attention",
              "attention_decode", "attention_prefill", "attention_prefill_shared", "argmax", "sample",
-             "add_deltas", "add_normed_rmsnorm", "act_mul_rows", "add_rows"]
+             "add_deltas", "add_normed_rmsnorm", "act_mul_rows", "add_rows", "embed_pairs", "qkv_store",
+             "latent_prepare", "rotate_heads", "latent_attention", "gemm_batched", "mlstm_scan", "headnorm_gate",
+             "xielu"]
     spans: list[tuple[str, object, object]] = []
     saved = {n: getattr(ops, n) for n in names}
 
@@ -399,20 +403,69 @@ def mofarax_like(qcfg, mask_size: int, side_dim: int):
     return mcfg, sizes
 
 
+def minilorn_like(qcfg, window: int, pattern: str):
+    """A Minilorn configuration with the layer sizes of a Qwen2 one (same width, feed-forward
+    width, vocabulary and number of layers): attention layers with Qwen2's heads (values as
+    large as keys); latent attention with as many heads, a query latent of 3/8 and a key/value
+    latent of 1/8 of the width (rounded to 64) and half a head rotated; matrix memories of
+    width / 512 heads with 256 query/key and 512 value elements; `pattern` says which mixer
+    each layer has, letter by letter (a, l, m), repeated.  With it an object that names the
+    sizes as the formulas of this program expect them."""
+    from types import SimpleNamespace
+
+    from shrike_amd.models.minilorn import (LatentAttention, MatrixMemory, MinilornConfig, MinilornLayer,
+                                            SinkAttention)
+
+    h, d, H = qcfg.hidden_size, qcfg.head_dim, qcfg.num_attention_heads
+    up64 = lambda x: max(64, -(-int(x) // 64) * 64)  # noqa: E731
+    mixers = {
+        "a": ("attention", SinkAttention(heads=H, kv_heads=qcfg.num_key_value_heads, dim=d, vdim=d, scale=d**-0.5,
+                                         softcap=50.0, q_temp=(0.5, 128))),
+        "l": ("latent_attention", LatentAttention(heads=H, dim=d, rot_dim=d // 2, vdim=d, q_rank=up64(3 * h / 8),
+                                                   kv_rank=up64(h / 8), scale=(1.5 * d) ** -0.5, rot_base=10000.0,
+                                                   window=window, rot_dims=d // 2)),
+        "m": ("mlstm", MatrixMemory(heads=max(1, h // 512), dim=256, vdim=512, gate_cap=15.0)),
+    }
+    kinds = [mixers[pattern[i % len(pattern)]] for i in range(qcfg.num_hidden_layers)]
+    layers = tuple(MinilornLayer(kind, mixer, qcfg.intermediate_size) for kind, mixer in kinds)
+    mcfg = MinilornConfig(vocab=qcfg.vocab_size, width=h, norm_eps=qcfg.rms_norm_eps, layers=layers,
+                          bigram=(65521, 31, 17))
+    la, mm = mixers["l"][1], mixers["m"][1]
+    elements = {
+        "attention": 2 * (H + qcfg.num_key_value_heads) * d * h,
+        "latent_attention": (la.q_rank + la.kv_rank + la.rot_dim) * h + H * (d + la.rot_dim) * la.q_rank
+        + 2 * H * d * la.kv_rank + H * d * h,
+        "mlstm": (2 * mm.heads * mm.dim + 3 * mm.heads * mm.vdim + 2 * mm.heads) * h,
+    }
+    cached = {"attention": 2 * qcfg.num_key_value_heads * d, "latent_attention": la.kv_rank + la.rot_dim, "mlstm": 0}
+    n = len(kinds)
+    sizes = SimpleNamespace(
+        hidden_size=h, head_dim=d, num_attention_heads=H, num_key_value_heads=qcfg.num_key_value_heads,
+        intermediate_size=qcfg.intermediate_size, num_hidden_layers=n, vocab_size=qcfg.vocab_size,
+        layer_elements=sum(elements[k] for k, _ in kinds) // n + 2 * h * qcfg.intermediate_size,
+        kv_elements_per_token=sum(cached[k] for k, _ in kinds))
+    return mcfg, sizes
+
+
 def run_designs(args, qcfg) -> dict:
-    """Mofarax beside Qwen2 at equal layer sizes, random weights: a prompt of 2,048 tokens
-    in one step, decode steps at batch 1, 8 and 64 from that context, and what each
+    """Another design beside Qwen2 at equal layer sizes, random weights: a prompt of 2,048
+    tokens in one step, decode steps at batch 1, 8 and 64 from that context, and what each
     kernel takes in a decode step at batch 8 and in the prompt's step."""
     import gc
 
     import torch
 
     from shrike_amd import SamplingParams
-    from shrike_amd.models import mofarax, qwen2
+    from shrike_amd.models import minilorn, mofarax, qwen2
 
-    mcfg, msizes = mofarax_like(qcfg, args.mask_size, args.side_dim)
+    if args.minilorn:
+        mcfg, msizes = minilorn_like(qcfg, args.window, args.pattern)
+        other = ("minilorn", minilorn.build_spec(mcfg), msizes)
+    else:
+        mcfg, msizes = mofarax_like(qcfg, args.mask_size, args.side_dim)
+        other = ("mofarax", mofarax.build_spec(mcfg), msizes)
     out = {}
-    for name, spec, sizes in (("qwen2", qwen2.build_spec(qcfg), qcfg), ("mofarax", mofarax.build_spec(mcfg), msizes)):
+    for name, spec, sizes in (("qwen2", qwen2.build_spec(qcfg), qcfg), other):
         if args.design_only and name != args.design_only:
             continue
         engine = make_engine(sizes, spec, 64, args.seed)
@@ -585,8 +638,14 @@ def main() -> int:
     ap.add_argument("--mofarax", action="store_true",
                     help="instead of the default run: the Mofarax design beside Qwen2 at the layer sizes of "
                          "--shape, random weights: prompt, decode at batch 1 / 8 / 64, per-kernel times")
-    ap.add_argument("--design-only", choices=["qwen2", "mofarax"], default=None,
-                    help="--mofarax: run only this one of the two (for a profile of one model's kernels)")
+    ap.add_argument("--minilorn", action="store_true",
+                    help="Minilorn beside Qwen2 at equal layer sizes: prompt, decode at batch 1/8/64, time per kernel")
+    ap.add_argument("--pattern", default="alml", metavar="LETTERS",
+                    help="--minilorn: the layers' mixers in order, repeated: a(ttention), l(atent attention), m(atrix memory)")
+    ap.add_argument("--window", type=int, default=4096, metavar="N",
+                    help="--minilorn: sliding window of its latent attention (4096: no fewer keys than Qwen2 reads)")
+    ap.add_argument("--design-only", choices=["qwen2", "mofarax", "minilorn"], default=None,
+                    help="--mofarax / --minilorn: run only this one of the two (for a profile of one model's kernels)")
     ap.add_argument("--mask-size", type=int, default=8192, metavar="N",
                     help="--mofarax: positions per block of its attention (8192: no fewer keys than Qwen2 reads)")
     ap.add_argument("--side-dim", type=int, default=256, metavar="N", help="--mofarax: width of its per-layer token input")
@@ -619,16 +678,19 @@ def main() -> int:
         raw["num_hidden_layers"] = args.layers
     cfg = Qwen2Config.from_dict(raw)
     spec = build_spec(cfg)
-    if args.mofarax:
+    if args.mofarax or args.minilorn:
         designs = run_designs(args, cfg)
+        design = "Minilorn" if args.minilorn else "Mofarax"
+        config = {"shape": args.shape, "layers": cfg.num_hidden_layers, "prompt": PROMPT_LEN,
+                  "decode_steps": args.design_steps}
+        config.update({"pattern": args.pattern, "window": args.window} if args.minilorn
+                      else {"mask_size": args.mask_size, "side_dim": args.side_dim})
         print(json.dumps({
-            "metric": f"Mofarax beside Qwen2 at the Qwen2.5-{args.shape.upper()} layer sizes: prompt tok/s, decode "
+            "metric": f"{design} beside Qwen2 at the Qwen2.5-{args.shape.upper()} layer sizes: prompt tok/s, decode "
                       "tok/s, us per kernel",
-            "value": designs[args.design_only or "mofarax"]["decode_b8"]["tok_s"], "unit": "tok/s", "n_gpus": 1, "higher_is_better": True,
+            "value": designs[args.design_only or design.lower()]["decode_b8"]["tok_s"], "unit": "tok/s", "n_gpus": 1, "higher_is_better": True,
             "dtype": "bf16", "data": "synthetic: random weights, prompt ids uniform in [0, vocab)",
-            "config": {"shape": args.shape, "layers": cfg.num_hidden_layers, "mask_size": args.mask_size,
-                       "side_dim": args.side_dim, "prompt": PROMPT_LEN, "decode_steps": args.design_steps},
-            "designs": designs}))
+            "config": config, "designs": designs}))
         return 0
     if args.products:
         products = run_products(cfg, [1, 8, 64, 512, PROMPT_LEN])

@@ -79,6 +79,21 @@ __device__ __forceinline__ float lanes4_sum(float v) {
   return bits_as_float(halves[0]) + bits_as_float(halves[1]);
 }
 
+// What a design may do to its scores beyond scaling them (the decode kernel and the
+// shared-key prompt kernel; scores are kept as base-2 logarithms there):
+//   cap_out != 0: s <- cap * tanh(s * scale / cap), formed as cap_out * (1 - 2 / (1 + 2^(s * cap_in)))
+//                 with cap_in = 2 * scale * log2(e) / cap and cap_out = cap * log2(e);
+//   sinks != null: one more term 2^(sinks[head] * log2(e)) in the head's denominator, which has
+//                 no key and no value (added where a row is normalised, or by the merge kernel).
+struct ScoreOpts {
+  float cap_in, cap_out;
+  const float* sinks;
+};
+
+__device__ __forceinline__ float capped_log2(float s, const ScoreOpts& so) {
+  return so.cap_out * (1.f - 2.f * __builtin_amdgcn_rcpf(1.f + __builtin_amdgcn_exp2f(s * so.cap_in)));
+}
+
 constexpr int kPStride = 40;  // bf16 elements per row of the P tile in LDS (32 + padding)
 
 // A window of 64 entries of a sequence's block table held across the lanes of
@@ -353,7 +368,7 @@ __global__ void __launch_bounds__(kDecodeWaves* kWave)
                             const int32_t* __restrict__ tables, int table_stride,
                             const bf16* __restrict__ k_pool, const bf16* __restrict__ v_pool,
                             int page_size, uint32_t page_magic, int window, int block, float scale,
-                            float* __restrict__ partial, int nsplit) {
+                            float* __restrict__ partial, int nsplit, ScoreOpts so) {
   constexpr int NBUF = 2;  // chunk buffers: one computed, one in flight
   constexpr int kStep = 32 * kDecodeWaves;  // keys between two chunks of one wavefront
   __shared__ float m_lds[kDecodeWaves][16], l_lds[kDecodeWaves][16];
@@ -448,6 +463,11 @@ __global__ void __launch_bounds__(kDecodeWaves* kWave)
       float sc[8];
 #pragma unroll
       for (int e = 0; e < 8; ++e) sc[e] = s[e / 4][e % 4] * scale2;
+      if (so.cap_out != 0.f) {  // (the same for every wavefront of the launch; kept a branch)
+        asm volatile("");
+#pragma unroll
+        for (int e = 0; e < 8; ++e) sc[e] = capped_log2(s[e / 4][e % 4], so);
+      }
       const int g0 = kb + g * 8;
       if (edge) {
 #pragma unroll
@@ -567,6 +587,7 @@ __global__ void __launch_bounds__(kDecodeWaves* kWave)
   const int head = kvh * group + j;
   if (nsplit == 1) {
     // the whole range in one wavefront: normalise and write the output row
+    if (so.sinks) l += __builtin_amdgcn_exp2f(so.sinks[head] * 1.4426950408889634f - m_ref);
     const float inv = 1.f / l;
     bf16* dst = out + (static_cast<size_t>(seq) * heads + head) * D + 4 * g;
 #pragma unroll
@@ -592,7 +613,8 @@ __global__ void __launch_bounds__(kDecodeWaves* kWave)
 // order.  One wavefront per (sequence, head); lane z holds split z's weight.
 template <int D>
 __global__ void __launch_bounds__(kWave)
-    attention_merge_kernel(const float* __restrict__ partial, bf16* __restrict__ out, int nsplit) {
+    attention_merge_kernel(const float* __restrict__ partial, bf16* __restrict__ out, int nsplit,
+                           const float* __restrict__ sinks, int heads) {
   constexpr int NE = (D + kWave - 1) / kWave;  // elements per lane
   constexpr int kBatch = 8;                    // splits in flight
   __shared__ float weight[kMaxSplits];
@@ -626,6 +648,8 @@ __global__ void __launch_bounds__(kWave)
   const float wl = w * mine.y;
   float den = 0.f;
   for (int zz = 0; zz < nsplit; ++zz) den += __shfl(wl, zz, kWave);
+  // a head's sink: one more term of the denominator, behind no split's values
+  if (sinks) den += __builtin_amdgcn_exp2f(sinks[row % heads] * 1.4426950408889634f - mx);
 
   float acc[NE];
 #pragma unroll
@@ -746,7 +770,7 @@ __global__ void __launch_bounds__(WAVES* kWave) __attribute__((amdgpu_waves_per_
                                     const bf16* __restrict__ k_pool, const bf16* __restrict__ v_pool,
                                     int page_size, uint32_t page_magic, int window, int block, float scale,
                                     float* __restrict__ partial, int nsplit, int first_token,
-                                    int partial_rows) {
+                                    int partial_rows, ScoreOpts so) {
   constexpr int U = kUnitsPerWave;
   constexpr int kKFrags = 2 * (D / 32), kVFrags = D / 16, kFrags = kKFrags + kVFrags;
   // fragments each wavefront stages; where they do not divide, some are staged twice
@@ -903,6 +927,11 @@ __global__ void __launch_bounds__(WAVES* kWave) __attribute__((amdgpu_waves_per_
       float sc[8];
 #pragma unroll
       for (int e = 0; e < 8; ++e) sc[e] = s[e / 4][e % 4] * scale2;
+      if (so.cap_out != 0.f) {  // (the same for every wavefront of the launch; kept a branch)
+        asm volatile("");
+#pragma unroll
+        for (int e = 0; e < 8; ++e) sc[e] = capped_log2(s[e / 4][e % 4], so);
+      }
       if (edge) {  // wave-uniform: some query of the workgroup does not read the whole chunk
         // (the empty statement keeps this a branch: turned into selects, the
         // comparisons would run for every chunk)
@@ -986,6 +1015,7 @@ __global__ void __launch_bounds__(WAVES* kWave) __attribute__((amdgpu_waves_per_
                                    (row * nsplit + z) * 2) = make_float2(m[u], total);
       continue;
     }
+    if (so.sinks) total += __builtin_amdgcn_exp2f(so.sinks[unit_head[u]] * 1.4426950408889634f - m[u]);
     const float inv = 1.f / total;
     bf16* dst = out + static_cast<size_t>(tok0 + unit_q0[u] + j) * heads * D +
                 static_cast<size_t>(unit_head[u]) * D + 4 * g;
@@ -1005,18 +1035,19 @@ template <int D>
 static void launch_decode(dim3 grid, hipStream_t s, const bf16* q, int q_stride, bf16* out,
                           int heads, int kv_heads, const int32_t* positions, const int32_t* tables,
                           int table_stride, const bf16* k_pool, const bf16* v_pool, int page_size,
-                          int window, int block, float scale, float* partial, int nsplit, int streaming) {
+                          int window, int block, float scale, float* partial, int nsplit, int streaming,
+                          ScoreOpts so) {
   const uint32_t magic = static_cast<uint32_t>(((1ull << 32) + page_size - 1) / page_size);
   if (streaming)
     attention_decode_kernel<D, true><<<grid, kDecodeWaves * kWave, 0, s>>>(
         q, q_stride, out, heads, kv_heads, positions, tables, table_stride, k_pool, v_pool, page_size,
-        magic, window, block, scale, partial, nsplit);
+        magic, window, block, scale, partial, nsplit, so);
   else
     attention_decode_kernel<D, false><<<grid, kDecodeWaves * kWave, 0, s>>>(
         q, q_stride, out, heads, kv_heads, positions, tables, table_stride, k_pool, v_pool, page_size,
-        magic, window, block, scale, partial, nsplit);
+        magic, window, block, scale, partial, nsplit, so);
   if (nsplit > 1)
-    attention_merge_kernel<D><<<grid.y * heads, kWave, 0, s>>>(partial, out, nsplit);
+    attention_merge_kernel<D><<<grid.y * heads, kWave, 0, s>>>(partial, out, nsplit, so.sinks, heads);
 }
 
 template <int D>
@@ -1038,22 +1069,28 @@ static void launch_prefill_shared(dim3 grid, hipStream_t s, const bf16* q, int q
                                   const int32_t* wg_q0, const int32_t* tables, int table_stride,
                                   const bf16* k_pool, const bf16* v_pool, int page_size, int window, int block,
                                   float scale, bool small, float* partial, int nsplit,
-                                  int first_token, int prompt_tokens) {
+                                  int first_token, int prompt_tokens, ScoreOpts so) {
   const uint32_t magic = static_cast<uint32_t>(((1ull << 32) + page_size - 1) / page_size);
   const int rows = prompt_tokens * heads;
   if (small)
     attention_prefill_shared_kernel<D, kSharedWavesSmall><<<grid, kSharedWavesSmall * kWave, 0, s>>>(
         q, q_stride, out, heads, kv_heads, tiles, cu_q, ctx_lens, wg_seq, wg_q0, tables,
         table_stride, k_pool, v_pool, page_size, magic, window, block, scale, partial, nsplit, first_token,
-        rows);
+        rows, so);
   else
     attention_prefill_shared_kernel<D, kSharedWaves><<<grid, kSharedWaves * kWave, 0, s>>>(
         q, q_stride, out, heads, kv_heads, tiles, cu_q, ctx_lens, wg_seq, wg_q0, tables,
         table_stride, k_pool, v_pool, page_size, magic, window, block, scale, partial, nsplit, first_token,
-        rows);
+        rows, so);
   if (nsplit > 1)
     attention_merge_kernel<D><<<rows, kWave, 0, s>>>(
-        partial, out + static_cast<size_t>(first_token) * heads * D, nsplit);
+        partial, out + static_cast<size_t>(first_token) * heads * D, nsplit, so.sinks, heads);
+}
+
+static ScoreOpts score_opts(float scale, float softcap, const float* sinks) {
+  const float log2e = 1.4426950408889634f;
+  if (softcap > 0.f) return ScoreOpts{2.f * scale * log2e / softcap, softcap * log2e, sinks};
+  return ScoreOpts{0.f, 0.f, sinks};
 }
 
 }  // namespace shk
@@ -1097,7 +1134,10 @@ extern "C" int shk_attention_decode_bf16(const void* q, int q_stride, void* out,
                                          const int32_t* positions, const int32_t* tables,
                                          int table_stride, const void* k_pool, const void* v_pool,
                                          int page_size, int window, int block, float scale, float* partial,
-                                         int nsplit, int streaming, void* stream) {
+                                         int nsplit, int streaming, float softcap, const float* sinks,
+                                         void* stream) {
+  SHK_REQUIRE(softcap >= 0.f, "attention_decode: a score cap must be positive (0: none), got %g", softcap);
+  const ScoreOpts so = score_opts(scale, softcap, sinks);
   if (check_mfma_shapes("attention_decode", heads, kv_heads, head_dim, page_size, q_stride)) return 1;
   SHK_REQUIRE(heads / kv_heads <= 16, "attention_decode: at most 16 query heads per key/value head");
   SHK_REQUIRE(num_seqs >= 0 && num_seqs <= 65535 && nsplit >= 1 && nsplit <= kMaxSplits,
@@ -1118,7 +1158,7 @@ extern "C" int shk_attention_decode_bf16(const void* q, int q_stride, void* out,
   launch_decode<D>(grid, s, static_cast<const bf16*>(q), q_stride, static_cast<bf16*>(out), heads, \
                    kv_heads, positions, tables, table_stride, static_cast<const bf16*>(k_pool),    \
                    static_cast<const bf16*>(v_pool), page_size, window, block, scale, partial, nsplit,    \
-                   streaming)
+                   streaming, so)
   SHK_DISPATCH_D(head_dim, CALL)
 #undef CALL
   SHK_LAUNCH_CHECK("attention_decode");
@@ -1142,7 +1182,10 @@ extern "C" int shk_attention_prefill_shared_bf16(const void* q, int q_stride, vo
                                                  int table_stride, const void* k_pool,
                                                  const void* v_pool, int page_size, int window, int block,
                                                  float scale, int small, float* partial, int nsplit,
-                                                 int first_token, int prompt_tokens, void* stream) {
+                                                 int first_token, int prompt_tokens, float softcap,
+                                                 const float* sinks, void* stream) {
+  SHK_REQUIRE(softcap >= 0.f, "attention_prefill_shared: a score cap must be positive (0: none), got %g", softcap);
+  const ScoreOpts so = score_opts(scale, softcap, sinks);
   if (check_mfma_shapes("attention_prefill_shared", heads, kv_heads, head_dim, page_size, q_stride))
     return 1;
   const int tiles = shk_attention_prefill_shared_tiles(heads, kv_heads, head_dim, small);
@@ -1173,7 +1216,7 @@ extern "C" int shk_attention_prefill_shared_bf16(const void* q, int q_stride, vo
                            heads, kv_heads, tiles, cu_q, ctx_lens, wg_seq, wg_q0, tables,      \
                            table_stride, static_cast<const bf16*>(k_pool),                     \
                            static_cast<const bf16*>(v_pool), page_size, window, block, scale, small != 0, \
-                           partial, nsplit, first_token, prompt_tokens)
+                           partial, nsplit, first_token, prompt_tokens, so)
   switch (head_dim) {
     case 32: CALL(32); break;
     case 64: CALL(64); break;

@@ -15,7 +15,7 @@ from ctypes import c_char_p, c_float, c_int, c_longlong, c_void_p
 
 _LIB = None
 _RECORDING: list | None = None  # (launcher id, argument tuple) while a step is being recorded
-CALL_MAX_ARGS = 26
+CALL_MAX_ARGS = 28
 
 
 class KernelError(RuntimeError):
@@ -55,11 +55,12 @@ _SIGNATURES = {
     "shk_xielu": [_P, _P, _I, c_longlong, _F, _F, _P],
     "shk_embed_pairs": [_P, _P, _I, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _P],
     "shk_attention_supports_mfma": [_I, _I, _I, _I, _I],
-    "shk_attention_decode_bf16": [_P, _I, _P, _I, _I, _I, _I, _P, _P, _I, _P, _P, _I, _I, _I, _F, _P, _I, _I, _P],
+    "shk_attention_decode_bf16": [_P, _I, _P, _I, _I, _I, _I, _P, _P, _I, _P, _P, _I, _I, _I, _F, _P, _I, _I, _F, _P,
+                                  _P],
     "shk_attention_prefill_bf16": [_P, _I, _P, _I, _I, _I, _I, _P, _P, _P, _P, _P, _I, _P, _P, _I, _I, _I, _F, _P],
     "shk_attention_prefill_shared_tiles": [_I, _I, _I, _I],
     "shk_attention_prefill_shared_bf16": [_P, _I, _P, _I, _I, _I, _I, _P, _P, _P, _P, _P, _I, _P, _P, _I, _I, _I, _F,
-                                          _I, _P, _I, _I, _I, _P],
+                                          _I, _P, _I, _I, _I, _F, _P, _P],
     "shk_argmax": [_P, _P, _I, _I, _I, _P, _P],
     "shk_argmax_scratch_floats": [_I, _I],
     "shk_sample": [_P, _P, _P, _P, _P, _P, c_longlong, _I, _I, _I, _I, _P],

@@ -667,8 +667,17 @@ def attention_supports_mfma(heads, kv_heads, head_dim, page_size, q_stride) -> b
     return bool(load().shk_attention_supports_mfma(heads, kv_heads, head_dim, page_size, q_stride))
 
 
+def _sinks(sinks, heads, who):
+    if sinks is None:
+        return None
+    if sinks.numel() != heads or not sinks.is_contiguous():
+        raise KernelError(f"{who}: sinks must hold one value per head ({heads})")
+    return _dev(sinks, "sinks", torch.float32)
+
+
 def attention_decode(q, out, num_seqs, heads, kv_heads, head_dim, positions, tables, k_pool, v_pool,
-                     page_size, window, scale, partial, nsplit, streaming=False, chunk=None) -> None:
+                     page_size, window, scale, partial, nsplit, streaming=False, chunk=None, softcap=None,
+                     sinks=None) -> None:
     """bfloat16 MFMA attention for the first num_seqs rows of q, one token per sequence.
     `streaming`: fetch keys and values with non-temporal loads (same result; faster when
     the launch reads tens of megabytes of them)."""
@@ -688,7 +697,7 @@ def attention_decode(q, out, num_seqs, heads, kv_heads, head_dim, positions, tab
             _dev(positions, "positions", torch.int32), _dev(tables, "tables", torch.int32),
             tables.shape[1], _dev(k_pool, "k_pool"), _dev(v_pool, "v_pool"), page_size,
             int(window or 0), int(chunk or 0), float(scale), _dev(partial, "partial", torch.float32), nsplit,
-            int(bool(streaming)), _stream(),
+            int(bool(streaming)), float(softcap or 0.0), _sinks(sinks, heads, "attention_decode"), _stream(),
         )
     )
 
@@ -723,7 +732,8 @@ def attention_prefill_shared_tiles(heads, kv_heads, head_dim, small=False) -> in
 
 def attention_prefill_shared(q, out, num_wgs, heads, kv_heads, head_dim, cu_q, ctx_lens, wg_seq, wg_q0,
                              tables, k_pool, v_pool, page_size, window, scale, small=False,
-                             partial=None, nsplit: int = 1, first_token: int = 0, chunk=None) -> None:
+                             partial=None, nsplit: int = 1, first_token: int = 0, chunk=None, softcap=None,
+                             sinks=None) -> None:
     """bfloat16 MFMA attention for prompt portions; one workgroup per (run of query
     tiles, key/value head) shares each chunk of keys among its query heads.
     wg_seq / wg_q0 are in steps of 16 * attention_prefill_shared_tiles(..., small),
@@ -752,7 +762,7 @@ def attention_prefill_shared(q, out, num_wgs, heads, kv_heads, head_dim, cu_q, c
             _dev(tables, "tables", torch.int32), tables.shape[1], _dev(k_pool, "k_pool"),
             _dev(v_pool, "v_pool"), page_size, int(window or 0), int(chunk or 0), float(scale), int(small),
             _dev(partial, "partial", torch.float32) if nsplit > 1 else None, int(nsplit), int(first_token),
-            int(prompt_tokens), _stream(),
+            int(prompt_tokens), float(softcap or 0.0), _sinks(sinks, heads, "attention_prefill_shared"), _stream(),
         )
     )
 

@@ -162,7 +162,9 @@ class PagedAttention(Mixer):
     def plain_store(self) -> bool:
         """Whether the step goes through the cache-write kernel without rotation that
         takes values of another size than keys, the queries' temperature and the
-        values' unit norm, and through the general attention kernel."""
+        values' unit norm (attention itself then runs on the matrix-instruction kernels
+        where they take the shape, values as large as keys included, else on the general
+        kernel)."""
         s = self.spec
         return bool(self.value_dim != s.head_dim or getattr(s, "query_temperature", None)
                     or getattr(s, "value_norm_eps", None) or getattr(s, "softcap", None)
@@ -258,8 +260,13 @@ class PagedAttention(Mixer):
         s = self.spec
         h, hkv, d = s.num_heads, s.num_kv_heads, s.head_dim
         plan = shape.notes[key] = AttentionPlan()
-        plan.mfma = self.dtype == torch.bfloat16 and not self.plain_store and ops.attention_supports_mfma(
+        plan.mfma = self.dtype == torch.bfloat16 and self.value_dim == d and ops.attention_supports_mfma(
             h, hkv, d, shape.page_size, self._qkv_width())
+        # capped scores and sinks are built into the decode kernel and the shared-key prompt
+        # kernel; where the latter does not take the shape, the general kernel serves the step
+        if plan.mfma and (getattr(s, "softcap", None) or getattr(s, "sinks", False)) \
+                and not ops.attention_prefill_shared_tiles(h, hkv, d):
+            plan.mfma = False
         # the most keys that any query reads, where the mask bounds them
         reach = min(x for x in (s.window, s.chunk, 1 << 40) if x)
         if not plan.mfma:
@@ -325,7 +332,8 @@ class PagedAttention(Mixer):
                                  torch.float32)
             ops.attention_decode(q, out, ctx.num_decode, h, hkv, d, ctx.positions, tables,
                                  cache.pools["k"], cache.pools["v"], cache.page_size, s.window, s.scale,
-                                 partial, plan.nsplit, plan.streaming, chunk=s.chunk)
+                                 partial, plan.nsplit, plan.streaming, chunk=s.chunk,
+                                 softcap=getattr(s, "softcap", None), sinks=self.sinks)
         if plan.kernel == "shared":
             partial = None
             if plan.portion_splits > 1:
@@ -337,7 +345,7 @@ class PagedAttention(Mixer):
                                          cache.pools["k"], cache.pools["v"], cache.page_size, s.window,
                                          s.scale, small=plan.small, partial=partial,
                                          nsplit=plan.portion_splits, first_token=plan.first_token,
-                                         chunk=s.chunk)
+                                         chunk=s.chunk, softcap=getattr(s, "softcap", None), sinks=self.sinks)
         elif plan.kernel == "tiles":
             ops.attention_prefill(q, out, plan.count, h, hkv, d, ctx.cu_q, ctx.ctx_lens,
                                   ctx.extras[plan.seq_name], ctx.extras[plan.q0_name], tables,

@@ -24,7 +24,8 @@ pytestmark = pytest.mark.gpu
 TOL = {"float32": 1e-4, "bfloat16": 1.5e-2}
 # lengths that end before, on and after the edges of the models' windows (9; 40 and 1;
 # none within reach; 17), of their query temperature's steps and of their pages
-LENGTHS = {"A": [1, 9, 49, 97, 130, 10], "B": [3, 41, 40, 29, 8, 150], "C": [2, 70, 33, 100], "D": [5, 34, 67, 120, 18]}
+LENGTHS = {"A": [1, 9, 49, 97, 130, 10], "B": [3, 41, 40, 29, 8, 150], "C": [2, 70, 33, 100], "D": [5, 34, 67, 120, 18],
+           "E": [700, 40, 330]}
 
 
 @pytest.fixture(scope="module")
@@ -49,7 +50,7 @@ def engine_parts(model_dir, dtype, page_size, pages, graphs=True, slots=4):
     return model, cache, ModelRunner(model, cache, rt, graphs=graphs)
 
 
-@pytest.mark.parametrize("name", ["A", "B", "C", "D"])
+@pytest.mark.parametrize("name", ["A", "B", "C", "D", "E"])
 def test_the_stream_after_every_layer(name, model_root):
     """float32: the residual stream after each layer against the plain model's, for a
     prompt that crosses window edges and steps of the query temperature."""
@@ -77,7 +78,8 @@ def test_the_stream_after_every_layer(name, model_root):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("name, page_size", [("A", 16), ("B", 4), ("B", 16), ("C", 32), ("D", 8), ("A", 8), ("D", 16)])
+@pytest.mark.parametrize("name, page_size", [("A", 16), ("B", 4), ("B", 16), ("C", 32), ("D", 8), ("A", 8), ("D", 16),
+                                             ("E", 16)])
 def test_four_cuttings_agree_with_the_plain_implementation(name, page_size, dtype, model_root, tmp_path):
     model_dir = make_model_dir(name, model_root, dtype=dtype)
     vocab = CONFIGS[name]["vocab"]
@@ -89,7 +91,10 @@ def test_four_cuttings_agree_with_the_plain_implementation(name, page_size, dtyp
     budget = max(-(-len(ids) // 64) * 64 for ids in seqs.values())
     whole(tb, "w_", seqs)
     last_one_by_one(tb, "d_", seqs, tail=45)
-    changing_portions(tb, "p_", seqs)
+    if name == "E":  # portions of hundreds of tokens far into a sequence: their keys are shared among workgroups
+        changing_portions(tb, "p_", seqs, sizes=(290, 2, 300, 7, 64, 1, 33))
+    else:
+        changing_portions(tb, "p_", seqs)
     mixed_budget = budget + 128
     mixed(tb, "m_", seqs, mixed_budget, seed=5)
     # four state slots: every request after the fourth takes one that another has held
@@ -235,6 +240,36 @@ def test_graphs_and_recorded_launches_equal_kernel_by_kernel_steps(dtype, model_
             assert runner.graph_replays > 0 and runner.list_replays > 0
         results.append(torch.cat(rows))
     assert torch.equal(results[0], results[1])
+
+
+def test_the_matrix_instruction_kernels_serve_attention_with_sinks_and_caps(model_root, monkeypatch):
+    """bfloat16, values as large as keys, head sizes 64 and 128: single tokens go to the decode
+    kernel (with key splits, whose merge adds the sink), portions to the shared-key kernel
+    (also with its keys split); the general kernel is not called for these layers."""
+    from shrike_amd.engine.runner import StepEntry
+    from shrike_amd.kernels import ops
+
+    model_dir = make_model_dir("E", model_root, dtype="bfloat16")
+    plain = PlainMinilorn(model_dir)
+    model, cache, runner = engine_parts(model_dir, "bfloat16", 16, 128, graphs=False)
+    calls = {"general": 0, "decode": [], "shared": []}
+    real = {n: getattr(ops, n) for n in ("attention", "attention_decode", "attention_prefill_shared")}
+    monkeypatch.setattr(ops, "attention", lambda *a, **k: (calls.__setitem__("general", calls["general"] + 1), real["attention"](*a, **k))[1])
+    monkeypatch.setattr(ops, "attention_decode", lambda *a, **k: (calls["decode"].append(a[14]), real["attention_decode"](*a, **k))[1])
+    monkeypatch.setattr(ops, "attention_prefill_shared",
+                        lambda *a, **k: (calls["shared"].append(k.get("nsplit", 1)), real["attention_prefill_shared"](*a, **k))[1])
+    ids = requests_for("E", [900], seed=8)["r0"]
+    want = plain.logits(ids)
+    seq = cache.new_sequence()
+    rows, p = [], 0
+    for n in (600, 280, 1, 1, 18):
+        cache.append(seq, p, n)
+        rows.append(runner.step([StepEntry(seq, ids[p : p + n], p, list(range(n)))]).cpu().clone())
+        p += n
+    err = (torch.cat(rows).double() - want).abs().amax(-1) / want.abs().max()
+    assert float((err > 1.5e-2).float().mean()) <= 0.03 and float(err.max()) <= 4.5e-2, float(err.max())
+    assert calls["general"] == 0 and len(calls["decode"]) == 4 and len(calls["shared"]) == 6
+    assert max(calls["decode"]) > 1 and max(calls["shared"]) > 1, "the keys were meant to be split"
 
 
 def test_a_state_slot_that_is_used_again_starts_from_nothing(model_root):

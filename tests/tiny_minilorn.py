@@ -80,9 +80,21 @@ MIN_D = {
     ],
 }
 
-CONFIGS = {"A": MIN_A, "B": MIN_B, "C": MIN_C, "D": MIN_D}
-SEEDS = {"A": 3, "B": 11, "C": 23, "D": 41}
-PAGE_SIZES = {"A": 16, "B": 4, "C": 32, "D": 8}
+# head sizes that the matrix-instruction attention kernels take (values as large as keys, 64
+# and 128, grouped and ungrouped), for prompts long enough that keys are shared among workgroups
+MIN_E = {
+    "architecture": "Minilorn", "vocab": 180, "width": 96, "embedding": _bigram(50, 11, 29), "norm": {"eps": 1e-5},
+    "layers": [
+        _with(_attn(8, 2, 64, 64, softcap=6.0, coef=0.3, every=50), 128),
+        _with(_mlstm(1, 24, 32, cap=9.0), None),
+        _with(_attn(4, 4, 128, 128, softcap=20.0, coef=0.2, every=300), 72),
+        _with(_latent(2, 12, 4, 16, 20, 28, 100, base=1000.0), 64),
+    ],
+}
+
+CONFIGS = {"A": MIN_A, "B": MIN_B, "C": MIN_C, "D": MIN_D, "E": MIN_E}
+SEEDS = {"A": 3, "B": 11, "C": 23, "D": 41, "E": 53}
+PAGE_SIZES = {"A": 16, "B": 4, "C": 32, "D": 8, "E": 16}
 
 
 def make_model_dir(name: str, root=None, dtype: str = "float32", mode: str = "unit") -> Path:
