@@ -75,6 +75,7 @@ const Launcher kLaunchers[] = {
     SHK_LAUNCHER(shk_latent_prepare),
     SHK_LAUNCHER(shk_rotate_heads),
     SHK_LAUNCHER(shk_latent_attention),
+    SHK_LAUNCHER(shk_latent_attention_bf16),
     SHK_LAUNCHER(shk_gemm_batched),
     SHK_LAUNCHER(shk_mlstm_scan),
     SHK_LAUNCHER(shk_headnorm_gate),

@@ -577,6 +577,36 @@ def latent_attention(q, out, heads, key_dim, v_dim, positions, token_seq, tables
         int(window or 0), int(chunk or 0), float(scale), _stream()))
 
 
+def latent_attention_supports_mfma(heads: int, key_dim: int, v_dim: int) -> bool:
+    return bool(load().shk_latent_attention_supports_mfma(heads, key_dim, v_dim))
+
+
+def latent_attention_mfma(q, out, heads, key_dim, v_dim, positions, token_seq, tables, pool, page_size, window,
+                          scale, chunk=None, partial=None, nsplit: int = 1) -> None:
+    """latent_attention on the matrix units (bfloat16).  nsplit > 1 shares each token's rows among
+    that many workgroups; partial: float32 scratch of n * heads * nsplit * (v_dim + 2)."""
+    n = q.shape[0]
+    if q.dtype != torch.bfloat16 or out.dtype != torch.bfloat16:
+        raise KernelError("latent_attention_mfma: bfloat16 only")
+    if tuple(q.shape) != (n, heads * key_dim) or not q.is_contiguous() or tuple(out.shape) != (n, heads * v_dim) \
+            or not out.is_contiguous():
+        raise KernelError("latent_attention_mfma: q [n, heads * key_dim] and out [n, heads * v_dim], contiguous")
+    if (pool.dim() != 3 or tuple(pool.shape[1:]) != (page_size, key_dim) or not pool.is_contiguous()
+            or pool.dtype != q.dtype or tables.dim() != 2 or not tables.is_contiguous()):
+        raise KernelError(f"latent_attention_mfma: the pool must be contiguous [pages, {page_size}, {key_dim}] bfloat16")
+    if positions.shape[0] < n or token_seq.shape[0] < n:
+        raise KernelError("latent_attention_mfma: positions / token_seq are shorter than q")
+    if nsplit > 1 and (partial is None or partial.dtype != torch.float32
+                       or partial.numel() < n * heads * nsplit * (v_dim + 2)):
+        raise KernelError("latent_attention_mfma: key splits need a float32 partial buffer of "
+                          f"{n * heads * nsplit * (v_dim + 2)} values")
+    check(load().shk_latent_attention_bf16(
+        _dev(q, "q"), _dev(out, "out"), n, heads, key_dim, v_dim, _dev(positions, "positions", torch.int32),
+        _dev(token_seq, "token_seq", torch.int32), _dev(tables, "tables", torch.int32), tables.shape[1],
+        _dev(pool, "pool"), page_size, pool.shape[0], int(window or 0), int(chunk or 0), float(scale),
+        _dev(partial, "partial", torch.float32) if nsplit > 1 else None, int(nsplit), _stream()))
+
+
 def gemm_batched(a, w, out, batch: int, a_step: int, out_step: int) -> None:
     """out[:, b*out_step : b*out_step + m] = a[:, b*a_step : b*a_step + k] @ w[b].T for b < batch;
     w [batch, m, k] contiguous; a and out 2-d with unit inner stride; all of one dtype."""

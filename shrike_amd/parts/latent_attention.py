@@ -5,6 +5,7 @@ from __future__ import annotations
 import torch
 
 from ..kernels import ops
+from .attention import compute_units
 from .base import PAGE, Mixer, PagedSpec, PageTensor, ParamSpec, register_mixer
 
 
@@ -70,9 +71,35 @@ class LatentAttention(Mixer):
         if s.window is not None and s.window < 1:
             raise ValueError(f"{self.name}: window must be positive, got {s.window}")
 
+    def prepare(self, shape) -> None:
+        """Among how many workgroups each token's rows are shared on the matrix-instruction
+        path: few tokens with thousands of rows each (single tokens of long sequences) would
+        leave most of the chip idle.  From the step's shape alone (token count and longest
+        context rounded up to powers of two), so that a graph's steps all decide alike."""
+        s = self.spec
+        key = ("latent_attention", s.num_heads, s.kv_rank, s.rot_dim, s.window, s.chunk)
+        if key in shape.notes:
+            return
+        nsplit = 1
+        if self.mfma:
+            tokens, reach = 1, int(shape.ctx_lens.max())
+            while tokens < shape.num_tokens:
+                tokens *= 2
+            for bound in (s.window, s.chunk):
+                if bound:
+                    reach = min(reach, bound)
+            keys = 64
+            while keys < reach:
+                keys *= 2
+            nsplit = max(1, min(2 * compute_units() // tokens, keys // 128, 64))
+        shape.notes[key] = nsplit
+        shape.launch_key.append((key, nsplit))
+
     def load(self, tensors, runtime):
         s = self.spec
         H = s.num_heads
+        self.mfma = runtime.dtype == torch.bfloat16 and ops.latent_attention_supports_mfma(
+            H, s.kv_rank + s.rot_dim, s.kv_rank)
         self.w_down = runtime.weight(torch.cat([tensors[self._t("dq")], tensors[self._t("dkv")]], dim=0))
         self.q_norm = tensors[self._t("dq.norm")]
         self.kv_norm = tensors[self._t("dkv.norm")]
@@ -113,8 +140,17 @@ class LatentAttention(Mixer):
         ops.rotate_heads(q, q_head, s.head_dim, folded, key_dim, s.kv_rank, H, s.rot_dim, self.inv_freq,
                          ctx.positions)
         mixed = ctx.buffer("latent_mixed", (n, H * s.kv_rank), ctx.dtype)
-        ops.latent_attention(folded, mixed, H, key_dim, s.kv_rank, ctx.positions, ctx.token_seq, tables,
-                             cache.pools["latent"], cache.page_size, s.window, s.scale, chunk=s.chunk)
+        if self.mfma:
+            nsplit = ctx.notes[("latent_attention", H, s.kv_rank, s.rot_dim, s.window, s.chunk)]
+            partial = None
+            if nsplit > 1:
+                partial = ctx.buffer("latent_partial", (n * H * nsplit * (s.kv_rank + 2),), torch.float32)
+            ops.latent_attention_mfma(folded, mixed, H, key_dim, s.kv_rank, ctx.positions, ctx.token_seq, tables,
+                                      cache.pools["latent"], cache.page_size, s.window, s.scale, chunk=s.chunk,
+                                      partial=partial, nsplit=nsplit)
+        else:
+            ops.latent_attention(folded, mixed, H, key_dim, s.kv_rank, ctx.positions, ctx.token_seq, tables,
+                                 cache.pools["latent"], cache.page_size, s.window, s.scale, chunk=s.chunk)
         heads_out = ctx.buffer("latent_heads", (n, H * s.value_dim), ctx.dtype)
         ops.gemm_batched(mixed, self.w_uv, heads_out, H, s.kv_rank, s.value_dim)
         return self.linear_deferred(ctx, "attn_proj", heads_out, self.w_o)

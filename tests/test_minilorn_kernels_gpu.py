@@ -261,7 +261,8 @@ def test_rotation_of_a_slice_of_every_head(ops, dtype):
 
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("heads, key_dim, v_dim, window, page_size", [(8, 144, 128, 72, 16), (3, 15, 11, 9, 4), (2, 304, 272, 40, 8),
-                                                                      (1, 32, 30, 1, 16), (4, 48, 40, 1000, 16)])
+                                                                      (1, 32, 30, 1, 16), (4, 48, 40, 1000, 16), (28, 512, 448, 100, 16),
+                                                                      (20, 576, 512, 33, 16), (17, 640, 640, 64, 32)])
 def test_latent_attention_at_the_windows_edges(ops, dtype, heads, key_dim, v_dim, window, page_size):
     """Rows of a portion and single tokens.  For chosen queries one key is made to stand out:
     the oldest key inside the window (its row must dominate) or the newest outside it (it
@@ -304,6 +305,15 @@ def test_latent_attention_at_the_windows_edges(ops, dtype, heads, key_dim, v_dim
             want[t, h] = w @ kr[:, :v_dim]
     assert torch.isfinite(out).all(), "a row outside the sequence's pages or its window was read"
     close(out.view(n, heads, v_dim), want, dtype)
+    if dtype == torch.bfloat16 and ops.latent_attention_supports_mfma(heads, key_dim, v_dim):
+        # the same on the matrix units, each token's rows taken by one workgroup and shared among three
+        for nsplit in (1, 3):
+            again = torch.full((n, heads * v_dim), float("nan"), dtype=dtype, device="cuda")
+            partial = torch.full((n * heads * nsplit * (v_dim + 2),), float("nan"), device="cuda")
+            ops.latent_attention_mfma(dev(q.reshape(n, heads * key_dim)), again, heads, key_dim, v_dim, positions, token_seq,
+                                      dev(tables), pool, page_size, window, scale, partial=partial, nsplit=nsplit)
+            assert torch.isfinite(again).all(), f"{nsplit} shares: a row outside the window or the pages was read"
+            close(again.view(n, heads, v_dim), want, dtype, f"matrix units, {nsplit} shares")
     assert window >= 300 or (any(inside for _, inside in marks) and any(not inside for _, inside in marks))
 
 
