@@ -322,7 +322,7 @@ def kernel_breakdown(engine, steps: int = 3, before_step=None) -> dict:
     names = ["embed", "add_rmsnorm", "act_mul", "gemm", "gemm_tiled_weight", "rope_kv_store", "attention",
              "attention_decode", "attention_prefill", "attention_prefill_shared", "argmax", "sample",
              "add_deltas", "add_normed_rmsnorm", "act_mul_rows", "add_rows", "embed_pairs", "qkv_store",
-             "latent_prepare", "rotate_heads", "latent_attention", "gemm_batched", "mlstm_scan", "headnorm_gate",
+             "latent_prepare", "rotate_heads", "latent_attention", "latent_attention_mfma", "gemm_batched", "mlstm_scan", "headnorm_gate",
              "xielu"]
     spans: list[tuple[str, object, object]] = []
     saved = {n: getattr(ops, n) for n in names}

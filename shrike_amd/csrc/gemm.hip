@@ -71,6 +71,42 @@ __global__ void __launch_bounds__(256)
   }
 }
 
+// A batch of products with few rows of a (single tokens): one wavefront per (product of the
+// batch, output feature) walks that weight row once, every lane a run of it, and forms the dot
+// products of up to 16 rows of a at a time; sums over the lanes in a fixed order.  Weight rows
+// are read whole and once, and thousands of wavefronts keep the memory busy, where the tiled
+// kernel's few workgroups would each walk a long k alone.
+constexpr int kSkinnyRows = 16;
+
+template <typename T>
+__global__ void __launch_bounds__(256)
+    gemm_batched_skinny_kernel(const T* __restrict__ a, const T* __restrict__ w, T* __restrict__ out, int n,
+                               int m, int k, int lda, int ldo, long long a_batch, long long w_batch,
+                               long long out_batch) {
+  const int lane = threadIdx.x % kWave;
+  const int row = blockIdx.x * (256 / kWave) + threadIdx.x / kWave;  // output feature
+  if (row >= m) return;
+  const int b = blockIdx.y;
+  const T* wr = w + b * w_batch + static_cast<size_t>(row) * k;
+  const T* ab = a + b * a_batch;
+  for (int n0 = 0; n0 < n; n0 += kSkinnyRows) {
+    float acc[kSkinnyRows];
+#pragma unroll
+    for (int r = 0; r < kSkinnyRows; ++r) acc[r] = 0.f;
+    for (int kk = lane; kk < k; kk += kWave) {
+      const float wv = to_float(wr[kk]);
+#pragma unroll
+      for (int r = 0; r < kSkinnyRows; ++r)
+        if (n0 + r < n) acc[r] = fmaf(to_float(ab[static_cast<size_t>(n0 + r) * lda + kk]), wv, acc[r]);
+    }
+#pragma unroll
+    for (int r = 0; r < kSkinnyRows; ++r) {
+      const float total = wave_sum(acc[r]);
+      if (lane == 0 && n0 + r < n) out[b * out_batch + static_cast<size_t>(n0 + r) * ldo + row] = from_float<T>(total);
+    }
+  }
+}
+
 template <typename TI, typename TO>
 static int launch_tiled(const void* a, const void* w, const float* bias, void* out, int n, int m,
                         int k, int lda, int ldo, int accumulate, hipStream_t s, int batch = 1,
@@ -126,7 +162,17 @@ extern "C" int shk_gemm_batched(const void* a, const void* w, void* out, int n, 
   SHK_REQUIRE(a && w && out, "gemm_batched: null pointer");
   SHK_REQUIRE((n + kTM - 1) / kTM <= 65535, "gemm_batched: too many rows (%d)", n);
   hipStream_t s = static_cast<hipStream_t>(stream);
-  if (dtype == kF32)
+  if (n <= 2 * kSkinnyRows) {
+    dim3 grid((m + 3) / 4, batch);
+    if (dtype == kF32)
+      gemm_batched_skinny_kernel<float><<<grid, 256, 0, s>>>(static_cast<const float*>(a), static_cast<const float*>(w),
+                                                             static_cast<float*>(out), n, m, k, lda, ldo, a_batch,
+                                                             w_batch, out_batch);
+    else
+      gemm_batched_skinny_kernel<bf16><<<grid, 256, 0, s>>>(static_cast<const bf16*>(a), static_cast<const bf16*>(w),
+                                                            static_cast<bf16*>(out), n, m, k, lda, ldo, a_batch,
+                                                            w_batch, out_batch);
+  } else if (dtype == kF32)
     launch_tiled<float, float>(a, w, nullptr, out, n, m, k, lda, ldo, 0, s, batch, a_batch, w_batch, out_batch);
   else
     launch_tiled<bf16, bf16>(a, w, nullptr, out, n, m, k, lda, ldo, 0, s, batch, a_batch, w_batch, out_batch);

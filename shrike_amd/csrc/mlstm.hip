@@ -7,116 +7,152 @@
 // with log gates i_t = cap tanh(x / cap) and f_t = logsigmoid(cap tanh(y / cap)) of the
 // gates' projections x, y (bias added here).  The state before position 0 is zero (m = 0).
 //
-// mlstm_scan_kernel: one wavefront per (sequence, head, 16 value columns).  A lane owns
-// one column and every fourth row of S in registers; a token costs dim / 4 multiply-adds
-// a lane for S and as many for the readout, whose four partial sums meet by two lane
-// swaps.  Tokens are staged eight at a time through LDS (queries, keys, the 16 values,
-// the gates) so that the recurrence never waits for global memory.  Every wavefront
-// keeps n and m for itself (its own copy in the state), so no two wavefronts share
-// anything that one of them writes.  Prompt portions and single tokens take this one
-// path: a token's result does not depend on how its sequence was cut into steps.
+// mlstm_scan_kernel: one wavefront per (sequence, head, 4 value columns), eight of them (32
+// columns) in a workgroup.  A lane owns one column and a run of dim / 16 rows of S in
+// registers; a token costs dim / 16 multiply-adds a lane for S and as many for the readout,
+// whose sixteen partial sums meet by four lane exchanges.  Narrow tiles make many wavefronts
+// (a head of 512 values: 128), so that every SIMD of the chip has work and the chain from
+// token to token is short.  Tokens are staged sixteen at a time through LDS (queries and keys
+// once for the workgroup's eight wavefronts, each tile's values, the gates), all loads of a
+// stage in flight together, so that the recurrence never waits for global memory.  Every
+// wavefront keeps n and m for itself (its own copy in the state), so no two wavefronts share
+// anything that one of them writes.  Prompt portions and single tokens take this one path: a
+// token's result does not depend on how its sequence was cut into steps.
 //
-// State of one (slot, layer): [heads][tiles][dim * 16 + dim + 1] floats, tiles =
-// ceil(v_dim / 16): the tile's columns of S row by row, then n, then m.
+// State of one (slot, layer): [heads][tiles][64 RPT + 16 RPT + 1] floats, tiles = ceil(v_dim /
+// 4), RPT = rows per lane (4, 8 or 16 for dim up to 64, 128, 256): S as the lanes hold it,
+// [RPT][64 lanes] (lane = 4 * row group + column, row = RPT * row group + i), so that a
+// wavefront's loads and stores are whole lines; then n [RPT][16 row groups]; then m.
 #include "api.h"
 #include "common.h"
 
 namespace shk {
 
-constexpr int kCols = 16;      // value columns per wavefront
-constexpr int kRowGroups = 4;  // lanes that share a column take every fourth row
-constexpr int kStage = 8;      // tokens staged at a time
+constexpr int kCols = 4;        // value columns per wavefront
+constexpr int kRowGroups = 16;  // lanes that share a column split the rows among them
+constexpr int kStage = 16;      // tokens staged at a time
+constexpr int kScanWaves = 8;   // wavefronts (tiles) per workgroup
+
+__host__ __device__ inline int scan_rpt(int dim) { return dim <= 64 ? 4 : dim <= 128 ? 8 : 16; }
 
 __device__ __forceinline__ float log_sigmoid(float x) {
   return x >= 0.f ? -log1pf(expf(-x)) : x - log1pf(expf(x));
 }
 
-template <int RPT>  // rows per lane: dim <= 4 * RPT
-__global__ void __launch_bounds__(kWave)
+template <int RPT>  // rows per lane, a multiple of 4: dim <= 16 * RPT
+__global__ void __launch_bounds__(kScanWaves* kWave)
     mlstm_scan_kernel(const float* __restrict__ proj, int ld, int q_off, int k_off, int v_off, int i_off,
                       int f_off, const float* __restrict__ i_bias, const float* __restrict__ f_bias, float cap,
-                      float q_scale, int heads, int dim, int v_dim, const int32_t* __restrict__ positions,
+                      float q_scale, int heads, int dim, int v_dim, int tiles, const int32_t* __restrict__ positions,
                       const int32_t* __restrict__ cu_q, const int32_t* __restrict__ slots,
                       float* __restrict__ state, long long slot_stride, float* __restrict__ out) {
-  __shared__ float qs[kStage][4 * RPT];
-  __shared__ float ks[kStage][4 * RPT];
-  __shared__ float vs[kStage][kCols];
+  constexpr int ROWS = kRowGroups * RPT;
+  constexpr int kThreads = kScanWaves * kWave;
+  constexpr int kPerTile = kWave * RPT + kRowGroups * RPT + 1;
+  constexpr int kLoads = (kStage * ROWS + kThreads - 1) / kThreads;  // staging loads a thread and operand
+  __shared__ __attribute__((aligned(16))) float qs[kStage][ROWS];
+  __shared__ __attribute__((aligned(16))) float ks[kStage][ROWS];
+  __shared__ float vs[kScanWaves][kStage][kCols];
   __shared__ float gi[kStage], gf[kStage];
 
-  const int tile = blockIdx.x, head = blockIdx.y, seq = blockIdx.z;
-  const int tiles = gridDim.x;
-  const int lane = threadIdx.x, col = lane % kCols, rg = lane / kCols;
+  const int head = blockIdx.y, seq = blockIdx.z;
+  const int tid = threadIdx.x, wave = tid / kWave, lane = tid % kWave;
+  const int tile = blockIdx.x * kScanWaves + wave;
+  const bool live = tile < tiles;  // (a workgroup's last wavefronts may have no tile; they keep the barriers)
+  const int col = lane % kCols, rg = lane / kCols;
   const int vcol = tile * kCols + col;
   const int first = cu_q[seq], last = cu_q[seq + 1];
-  const int per_tile = dim * kCols + dim + 1;
   float* st = state + static_cast<size_t>(slots[seq]) * slot_stride +
-              (static_cast<size_t>(head) * tiles + tile) * per_tile;
+              (static_cast<size_t>(head) * tiles + (live ? tile : 0)) * kPerTile;
 
   float S[RPT], nv[RPT], m = 0.f;
   const bool fresh = positions[first] == 0;  // nothing precedes position 0
 #pragma unroll
   for (int i = 0; i < RPT; ++i) {
-    const int r = rg + kRowGroups * i;
-    const bool have = !fresh && r < dim;
-    S[i] = have ? st[r * kCols + col] : 0.f;
-    nv[i] = have ? st[dim * kCols + r] : 0.f;
+    const bool have = !fresh && live;
+    S[i] = have ? st[i * kWave + lane] : 0.f;
+    nv[i] = have ? st[kWave * RPT + i * kRowGroups + rg] : 0.f;
   }
-  if (!fresh) m = st[dim * kCols + dim];
+  if (!fresh && live) m = st[kPerTile - 1];
 
   for (int t0 = first; t0 < last; t0 += kStage) {
     const int count = last - t0 < kStage ? last - t0 : kStage;
-    __syncthreads();  // the tokens staged before have been read
-    for (int idx = lane; idx < count * 4 * RPT; idx += kWave) {
-      const int tt = idx / (4 * RPT), r = idx % (4 * RPT);
-      const float* row = proj + static_cast<size_t>(t0 + tt) * ld + head * dim;
-      qs[tt][r] = r < dim ? row[q_off + r] * q_scale : 0.f;
-      ks[tt][r] = r < dim ? row[k_off + r] : 0.f;
+    // the stage's queries and keys: every load issued before the first is used
+    float qv[kLoads], kv[kLoads];
+#pragma unroll
+    for (int u = 0; u < kLoads; ++u) {
+      const int idx = tid + u * kThreads;
+      const int tt = idx / ROWS, r = idx % ROWS;
+      const bool have = tt < count && r < dim;
+      const float* row = proj + static_cast<size_t>(t0 + (tt < count ? tt : 0)) * ld + head * dim + (r < dim ? r : 0);
+      qv[u] = have ? row[q_off] : 0.f;
+      kv[u] = have ? row[k_off] : 0.f;
     }
-    for (int idx = lane; idx < count * kCols; idx += kWave) {
-      const int tt = idx / kCols, c = idx % kCols;
+    float vv = 0.f;
+    {
+      const int tt = lane / kCols, c = lane % kCols;  // 16 tokens x 4 columns: one element a lane
       const int vc = tile * kCols + c;
-      vs[tt][c] = vc < v_dim ? proj[static_cast<size_t>(t0 + tt) * ld + v_off + head * v_dim + vc] : 0.f;
+      if (live && tt < count && vc < v_dim)
+        vv = proj[static_cast<size_t>(t0 + tt) * ld + v_off + head * v_dim + vc];
     }
-    if (lane < count) {
-      const float* row = proj + static_cast<size_t>(t0 + lane) * ld;
-      const float x = row[i_off + head] + i_bias[head], y = row[f_off + head] + f_bias[head];
-      gi[lane] = cap * tanhf(x / cap);
-      gf[lane] = log_sigmoid(cap * tanhf(y / cap));
+    float gx = 0.f, gy = 0.f;
+    if (tid < count) {
+      const float* row = proj + static_cast<size_t>(t0 + tid) * ld;
+      gx = row[i_off + head] + i_bias[head];
+      gy = row[f_off + head] + f_bias[head];
+    }
+    __syncthreads();  // the tokens staged before have been read
+#pragma unroll
+    for (int u = 0; u < kLoads; ++u) {
+      const int idx = tid + u * kThreads;
+      if (idx < kStage * ROWS) {
+        qs[idx / ROWS][idx % ROWS] = qv[u] * q_scale;
+        ks[idx / ROWS][idx % ROWS] = kv[u];
+      }
+    }
+    vs[wave][lane / kCols][lane % kCols] = vv;
+    if (tid < count) {
+      gi[tid] = cap * tanhf(gx / cap);
+      gf[tid] = log_sigmoid(cap * tanhf(gy / cap));
     }
     __syncthreads();
+    if (!live) continue;
     for (int tt = 0; tt < count; ++tt) {
       const float i_log = gi[tt], f_log = gf[tt];
       const float m_new = fmaxf(f_log + m, i_log);
       const float keep = expf(f_log + m - m_new), take = expf(i_log - m_new);
-      const float tv = take * vs[tt][col];
+      const float tv = take * vs[wave][tt][col];
       float o = 0.f, nq = 0.f;
 #pragma unroll
-      for (int i = 0; i < RPT; ++i) {
-        const int r = rg + kRowGroups * i;
-        const float kr = ks[tt][r], qr = qs[tt][r];
-        S[i] = fmaf(keep, S[i], kr * tv);
-        nv[i] = fmaf(keep, nv[i], take * kr);
-        o = fmaf(S[i], qr, o);
-        nq = fmaf(nv[i], qr, nq);
+      for (int i4 = 0; i4 < RPT; i4 += 4) {
+        const float4 k4 = *reinterpret_cast<const float4*>(&ks[tt][rg * RPT + i4]);
+        const float4 q4 = *reinterpret_cast<const float4*>(&qs[tt][rg * RPT + i4]);
+        const float kr[4] = {k4.x, k4.y, k4.z, k4.w}, qr[4] = {q4.x, q4.y, q4.z, q4.w};
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+          S[i4 + u] = fmaf(keep, S[i4 + u], kr[u] * tv);
+          nv[i4 + u] = fmaf(keep, nv[i4 + u], take * kr[u]);
+          o = fmaf(S[i4 + u], qr[u], o);
+          nq = fmaf(nv[i4 + u], qr[u], nq);
+        }
       }
-      o += __shfl_xor(o, 16, kWave);
-      o += __shfl_xor(o, 32, kWave);
-      nq += __shfl_xor(nq, 16, kWave);
-      nq += __shfl_xor(nq, 32, kWave);
+#pragma unroll
+      for (int off = kCols; off < kWave; off <<= 1) {  // over the sixteen lanes of a column, in a fixed order
+        o += __shfl_xor(o, off, kWave);
+        nq += __shfl_xor(nq, off, kWave);
+      }
       m = m_new;
       const float den = fmaxf(fabsf(nq), expf(-m)) + 1e-6f;
       if (rg == 0 && vcol < v_dim) out[static_cast<size_t>(t0 + tt) * heads * v_dim + head * v_dim + vcol] = o / den;
     }
   }
+  if (!live) return;
 #pragma unroll
   for (int i = 0; i < RPT; ++i) {
-    const int r = rg + kRowGroups * i;
-    if (r < dim) {
-      st[r * kCols + col] = S[i];
-      if (col == 0) st[dim * kCols + r] = nv[i];
-    }
+    st[i * kWave + lane] = S[i];
+    if (col == 0) st[kWave * RPT + i * kRowGroups + rg] = nv[i];
   }
-  if (lane == 0) st[dim * kCols + dim] = m;
+  if (lane == 0) st[kPerTile - 1] = m;
 }
 
 // out[t, h, :] = o[t, h, :] / rms(o[t, h, :]) * weight[h, :] * sigmoid(gate[t, h, :]): the
@@ -148,7 +184,8 @@ __global__ void __launch_bounds__(256)
 using namespace shk;
 
 extern "C" long long shk_mlstm_state_floats(int heads, int dim, int v_dim) {
-  return static_cast<long long>(heads) * ((v_dim + kCols - 1) / kCols) * (static_cast<long long>(dim) * kCols + dim + 1);
+  const int rpt = scan_rpt(dim);
+  return static_cast<long long>(heads) * ((v_dim + kCols - 1) / kCols) * (kWave * rpt + kRowGroups * rpt + 1);
 }
 
 extern "C" int shk_mlstm_scan(const float* proj, int ld, int q_off, int k_off, int v_off, int i_off, int f_off,
@@ -170,15 +207,17 @@ extern "C" int shk_mlstm_scan(const float* proj, int ld, int q_off, int k_off, i
   SHK_REQUIRE(num_seqs <= 65535 && heads <= 65535, "mlstm_scan: at most 65535 sequences and heads a call");
   SHK_REQUIRE(proj && i_bias && f_bias && positions && cu_q && slots && state && out, "mlstm_scan: null pointer");
   hipStream_t s = static_cast<hipStream_t>(stream);
-  dim3 grid((v_dim + kCols - 1) / kCols, heads, num_seqs);
-#define SHK_SCAN(R)                                                                                              \
-  mlstm_scan_kernel<R><<<grid, kWave, 0, s>>>(proj, ld, q_off, k_off, v_off, i_off, f_off, i_bias, f_bias, cap, \
-                                              q_scale, heads, dim, v_dim, positions, cu_q, slots, state,       \
-                                              slot_stride, out)
-  if (dim <= 32) SHK_SCAN(8);
-  else if (dim <= 64) SHK_SCAN(16);
-  else if (dim <= 128) SHK_SCAN(32);
-  else SHK_SCAN(64);
+  const int tiles = (v_dim + kCols - 1) / kCols;
+  dim3 grid((tiles + kScanWaves - 1) / kScanWaves, heads, num_seqs);
+#define SHK_SCAN(R)                                                                                          \
+  mlstm_scan_kernel<R><<<grid, kScanWaves * kWave, 0, s>>>(proj, ld, q_off, k_off, v_off, i_off, f_off, i_bias, \
+                                                           f_bias, cap, q_scale, heads, dim, v_dim, tiles,      \
+                                                           positions, cu_q, slots, state, slot_stride, out)
+  switch (scan_rpt(dim)) {
+    case 4: SHK_SCAN(4); break;
+    case 8: SHK_SCAN(8); break;
+    default: SHK_SCAN(16); break;
+  }
 #undef SHK_SCAN
   SHK_LAUNCH_CHECK("mlstm_scan");
   return 0;

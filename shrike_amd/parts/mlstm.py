@@ -37,11 +37,13 @@ class MatrixLSTM(Mixer):
         ]
 
     def state_floats(self) -> int:
-        """Per head and tile of 16 value columns: the tile's columns of S, then n and m
-        (every tile keeps its own copy of n and m; csrc/mlstm.hip)."""
+        """Per head and tile of 4 value columns: the tile's columns of S as the scan's lanes
+        hold them (rows padded to 64, 128 or 256), then n and m (every tile keeps its own
+        copy of n and m; csrc/mlstm.hip)."""
         s = self.spec
-        tiles = -(-s.value_dim // 16)
-        return s.num_heads * tiles * (s.head_dim * 16 + s.head_dim + 1)
+        tiles = -(-s.value_dim // 4)
+        rpt = 4 if s.head_dim <= 64 else 8 if s.head_dim <= 128 else 16
+        return s.num_heads * tiles * (64 * rpt + 16 * rpt + 1)
 
     def cache_spec(self):
         return StateSpec((self.state_floats(),), "float32")

@@ -318,7 +318,8 @@ def test_latent_attention_at_the_windows_edges(ops, dtype, heads, key_dim, v_dim
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("n, batch, m, k", [(1, 8, 128, 32), (70, 3, 10, 24), (5, 2, 65, 130)])
+@pytest.mark.parametrize("n, batch, m, k", [(1, 8, 128, 32), (70, 3, 10, 24), (5, 2, 65, 130), (32, 4, 7, 300), (33, 2, 64, 64),
+                                            (17, 28, 448, 128)])
 def test_batched_product(ops, dtype, n, batch, m, k):
     torch.manual_seed(7)
     a_step, out_step = k + 3, m + 5
