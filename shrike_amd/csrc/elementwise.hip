@@ -650,12 +650,41 @@ __global__ void xielu_kernel(const T* __restrict__ x, T* __restrict__ out, long 
 }
 }  // namespace shk
 
+namespace shk {
+// eight bfloat16 values a thread (16 bytes in, 16 bytes out)
+__global__ void xielu_vec_kernel(const uint4* __restrict__ x, uint4* __restrict__ out, long long vecs, float a_pos,
+                                 float a_neg) {
+  const long long i = static_cast<long long>(blockIdx.x) * blockDim.x + threadIdx.x;
+  if (i >= vecs) return;
+  const uint4 raw = x[i];
+  const uint32_t w[4] = {raw.x, raw.y, raw.z, raw.w};
+  uint32_t r[4];
+#pragma unroll
+  for (int e = 0; e < 4; ++e) {
+    float z[2] = {__uint_as_float(w[e] << 16), __uint_as_float(w[e] & 0xffff0000u)};
+#pragma unroll
+    for (int h = 0; h < 2; ++h)
+      z[h] = z[h] > 0.f ? fmaf(a_pos * z[h], z[h], 0.5f * z[h]) : fmaf(a_neg, expm1f(z[h]) - z[h], 0.5f * z[h]);
+    r[e] = bf16_bits(z[0]) | (static_cast<uint32_t>(bf16_bits(z[1])) << 16);
+  }
+  out[i] = make_uint4(r[0], r[1], r[2], r[3]);
+}
+}  // namespace shk
+
 extern "C" int shk_xielu(const void* x, void* out, int dtype, long long numel, float a_pos, float a_neg, void* stream) {
   SHK_REQUIRE(dtype == kF32 || dtype == kBF16, "xielu: unknown dtype %d", dtype);
   SHK_REQUIRE(numel >= 0 && numel < (1LL << 31) * 256, "xielu: bad size %lld", numel);
   if (numel == 0) return 0;
   SHK_REQUIRE(x && out, "xielu: null pointer");
   hipStream_t s = static_cast<hipStream_t>(stream);
+  if (dtype == kBF16 && numel % 8 == 0 && reinterpret_cast<uintptr_t>(x) % 16 == 0 &&
+      reinterpret_cast<uintptr_t>(out) % 16 == 0) {
+    const long long vecs = numel / 8;
+    shk::xielu_vec_kernel<<<static_cast<unsigned>((vecs + 255) / 256), 256, 0, s>>>(
+        static_cast<const uint4*>(x), static_cast<uint4*>(out), vecs, a_pos, a_neg);
+    SHK_LAUNCH_CHECK("xielu");
+    return 0;
+  }
   const unsigned grid = static_cast<unsigned>((numel + 255) / 256);
   if (dtype == kF32)
     shk::xielu_kernel<float><<<grid, 256, 0, s>>>(static_cast<const float*>(x), static_cast<float*>(out), numel, a_pos, a_neg);

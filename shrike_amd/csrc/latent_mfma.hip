@@ -1,7 +1,7 @@
 // bfloat16 attention through latents on the matrix units (gfx950).
 //
-// One workgroup per (token, share of its keys); wavefront w serves query heads 16 w .. 16 w + 15
-// of the token, a lane owns one head.  All heads read the same rows (one per cached token:
+// One workgroup of four wavefronts per (token, share of its keys, 64 heads); wavefront w serves 16
+// query heads of the token, a lane owns one head (wavefronts without heads help to stage the rows).  All heads read the same rows (one per cached token:
 // latent, then rotated key part), so a chunk of 32 rows is staged once per workgroup in LDS and
 // every wavefront takes both operands from there:
 //
@@ -11,7 +11,7 @@
 //                   rows' scores of its head, so P^T is already in B-operand layout
 //   O^T += V^T P^T  [v_dim x 16 heads]; the values are the rows' first v_dim elements, read
 //                   transposed out of LDS (8 rows' element d: eight 2-byte reads; rows are
-//                   padded by 32 bytes so that the four row groups fall into different banks)
+//                   padded and groups of 8 rows shifted so that these reads meet no bank twice)
 //
 // With nsplit > 1 the token's chunks are shared among nsplit workgroups, whose unnormalised
 // results (O, maximum, sum) latent_merge_kernel joins in order (single tokens with thousands
@@ -24,6 +24,7 @@ namespace shk {
 
 typedef __bf16 lbf16x8 __attribute__((ext_vector_type(8)));
 typedef float lf32x4 __attribute__((ext_vector_type(4)));
+typedef unsigned int lu32x4 __attribute__((ext_vector_type(4)));
 
 union LFrag {
   uint4 u;
@@ -40,14 +41,23 @@ __device__ __forceinline__ float quad_lanes_sum(float v) {
   return v + __shfl_xor(v, 32, kWave);
 }
 
+constexpr int kLatentWaves = 4;  // one wavefront a SIMD: each may hold the registers of 16 heads' sums
+
 template <int KS, int DB>  // rows of up to 32 KS elements, values of up to 16 DB
-__global__ void __launch_bounds__(512)
+__global__ void __launch_bounds__(kLatentWaves* kWave)
     latent_attention_mfma_kernel(const bf16* __restrict__ q, bf16* __restrict__ out, int heads, int key_dim,
                                  int v_dim, const int32_t* __restrict__ positions,
                                  const int32_t* __restrict__ token_seq, const int32_t* __restrict__ tables,
                                  int table_stride, const bf16* __restrict__ pool, int page_size, int num_pages,
                                  int window, int chunk, float scale, float* __restrict__ partial, int nsplit) {
-  constexpr int STRIDE = KS * 32 + 16;  // elements between rows in LDS
+  // Rows in LDS: KS * 32 elements and 64 bytes of padding (consecutive rows start 16 banks apart: the
+  // sixteen rows x four 16-byte pieces of a score operand cover the banks evenly), and every group of 8
+  // rows is shifted by 32 bytes more (the four groups that a transposed value read touches at once,
+  // 32 bytes each, fall into different banks).
+  constexpr int STRIDE = KS * 32 + 32;
+  auto at = [](int kk) { return kk * STRIDE + (kk >> 3) * 16; };
+  // 16-byte pieces of a chunk that a thread stages: 32 rows of at most 4 KS pieces, 256 threads
+  constexpr int kPieces = (32 * 4 * KS + kLatentWaves * kWave - 1) / (kLatentWaves * kWave);
   extern __shared__ __attribute__((aligned(16))) uint16_t rows[];  // [32][STRIDE]
   const int t = blockIdx.x, z = blockIdx.y;
   const int tid = threadIdx.x, nthreads = blockDim.x;
@@ -55,7 +65,7 @@ __global__ void __launch_bounds__(512)
   const int pos = positions[t];
   const int lo = first_key(pos, window, chunk);
   const int32_t* table = tables + static_cast<size_t>(token_seq[t]) * table_stride;
-  const int head = wave * 16 + j;
+  const int head = (blockIdx.z * kLatentWaves + wave) * 16 + j;  // (more than 64 heads: several workgroups a token)
   const bool col_ok = head < heads;
 
   // the queries of this wavefront's heads as B operands: head j, elements 32 ks + 8 g ..
@@ -68,7 +78,7 @@ __global__ void __launch_bounds__(512)
     if (col_ok && d0 < key_dim) qf[ks].u = *reinterpret_cast<const uint4*>(qrow + d0);
   }
   // what lies behind a row's elements stays zero for the whole kernel
-  for (int i = tid; i < 32 * STRIDE / 8; i += nthreads) reinterpret_cast<uint4*>(rows)[i] = make_uint4(0, 0, 0, 0);
+  for (int i = tid; i < (32 * STRIDE + 64) / 8; i += nthreads) reinterpret_cast<uint4*>(rows)[i] = make_uint4(0, 0, 0, 0);
   __syncthreads();
 
   const int key_begin = lo & ~31;
@@ -84,22 +94,52 @@ __global__ void __launch_bounds__(512)
 #pragma unroll
   for (int db = 0; db < DB; ++db) o[db] = lf32x4{0.f, 0.f, 0.f, 0.f};
 
+  // A chunk's rows travel in two steps: global memory to registers (all of a thread's pieces
+  // requested together, the next chunk's while this one is multiplied), registers to LDS.
+  // Rows that the token does not read are zero.
+  // (which row and which piece of it a thread stages does not change from chunk to chunk, and a
+  // division by a number that only the launch knows costs dozens of instructions: once, up here)
+  uint4 staged[kPieces];
+  int piece_row[kPieces], piece_col[kPieces], piece_lds[kPieces];
+#pragma unroll
+  for (int u = 0; u < kPieces; ++u) {
+    const int idx = tid + u * nthreads;
+    piece_row[u] = idx < 32 * npieces ? idx / npieces : -1;
+    piece_col[u] = (idx % npieces) * 8;
+    piece_lds[u] = at(piece_row[u] < 0 ? 0 : piece_row[u]) + piece_col[u];
+  }
+  const int page_shift = (page_size & (page_size - 1)) == 0 ? __ffs(page_size) - 1 : -1;
+  auto fetch = [&](int c) {
+    const int kb = key_begin + c * 32;
+#pragma unroll
+    for (int u = 0; u < kPieces; ++u) {
+      const int key = kb + piece_row[u];
+      staged[u] = make_uint4(0, 0, 0, 0);
+      if (piece_row[u] >= 0 && key >= lo && key <= pos) {
+        const int entry = page_shift >= 0 ? key >> page_shift : key / page_size;
+        const int slot = page_shift >= 0 ? key & (page_size - 1) : key % page_size;
+        const int page = table[entry];
+        if (page >= 0 && page < num_pages)
+          staged[u] = *reinterpret_cast<const uint4*>(
+              pool + (static_cast<size_t>(page) * page_size + slot) * key_dim + piece_col[u]);
+      }
+    }
+  };
+  auto put = [&]() {
+#pragma unroll
+    for (int u = 0; u < kPieces; ++u)
+      if (piece_row[u] >= 0) *reinterpret_cast<uint4*>(rows + piece_lds[u]) = staged[u];
+  };
+  if (c_first < c_end) fetch(c_first);
   for (int c = c_first; c < c_end; ++c) {
     const int kb = key_begin + c * 32;
-    // ---- the chunk's rows into LDS, 16 bytes a thread; rows that the token does not read are zero
-    for (int idx = tid; idx < 32 * npieces; idx += nthreads) {
-      const int kk = idx / npieces, piece = idx % npieces;
-      const int key = kb + kk;
-      uint4 v = make_uint4(0, 0, 0, 0);
-      if (key >= lo && key <= pos) {
-        const int page = table[key / page_size];
-        if (page >= 0 && page < num_pages)
-          v = *reinterpret_cast<const uint4*>(pool + (static_cast<size_t>(page) * page_size + key % page_size) * key_dim +
-                                              piece * 8);
-      }
-      *reinterpret_cast<uint4*>(rows + kk * STRIDE + piece * 8) = v;
-    }
+    put();
     __syncthreads();
+    if (c + 1 < c_end) fetch(c + 1);  // (the same for every thread of the workgroup)
+    if (head - j >= heads) {  // a wavefront that only helps to stage
+      __syncthreads();
+      continue;
+    }
 
     // ---- S^T for two tiles of 16 rows.  Row i of tile tt is row 8 (i / 4) + 4 tt + i % 4 of the
     // chunk, so that the lane's eight scores (4 tt + r) belong to the consecutive rows 8 g + e.
@@ -111,7 +151,7 @@ __global__ void __launch_bounds__(512)
 #pragma unroll
       for (int ks = 0; ks < KS; ++ks) {
         LFrag a;
-        a.u = *reinterpret_cast<const uint4*>(rows + kk * STRIDE + ks * 32 + g * 8);
+        a.u = *reinterpret_cast<const uint4*>(rows + at(kk) + ks * 32 + g * 8);
         s[tt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a.v, qf[ks].v, s[tt], 0, 0, 0);
       }
     }
@@ -135,13 +175,21 @@ __global__ void __launch_bounds__(512)
 #pragma unroll
     for (int e = 0; e < 8; ++e) pf.v[e] = static_cast<__bf16>(pr[e]);
     // ---- O^T += V^T P^T: A = element 16 db + j of rows 8 g .. 8 g + 7, B = the lane's own weights
+    if (__builtin_amdgcn_ballot_w64(alpha != 1.f) != 0) {  // some head's maximum rose
+#pragma unroll
+      for (int db = 0; db < DB; ++db) o[db] *= alpha;
+    }
+    const uint16_t* mine = rows + at(8 * g) + j;  // rows 8 g .. 8 g + 7 lie STRIDE apart
 #pragma unroll
     for (int db = 0; db < DB; ++db) {
-      LFrag vf;
+      // (packed by hand into a native vector: halves written one by one into a union's array
+      // would travel through scratch memory)
+      lu32x4 vw;
 #pragma unroll
-      for (int e = 0; e < 8; ++e) vf.h[e] = rows[(8 * g + e) * STRIDE + db * 16 + j];
-      o[db] *= alpha;
-      o[db] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf.v, pf.v, o[db], 0, 0, 0);
+      for (int e2 = 0; e2 < 4; ++e2)
+        vw[e2] = static_cast<uint32_t>(mine[(2 * e2) * STRIDE + db * 16]) |
+                 (static_cast<uint32_t>(mine[(2 * e2 + 1) * STRIDE + db * 16]) << 16);
+      o[db] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(lbf16x8, vw), pf.v, o[db], 0, 0, 0);
     }
     __syncthreads();  // the next chunk overwrites the rows
   }
@@ -162,7 +210,7 @@ __global__ void __launch_bounds__(512)
     return;
   }
   // a share's result: O [row][share][v_dim], then (maximum, sum) [row][share][2]
-  const size_t all_rows = static_cast<size_t>(gridDim.x) * heads;
+  const size_t all_rows = static_cast<size_t>(gridDim.x) * heads;  // (gridDim.x: the step's tokens)
   float* dst = partial + (row * nsplit + z) * v_dim;
 #pragma unroll
   for (int db = 0; db < DB; ++db)
@@ -203,12 +251,12 @@ __global__ void __launch_bounds__(kWave)
 }
 
 template <int KS, int DB>
-static void launch_latent(dim3 grid, int waves, hipStream_t s, const bf16* q, bf16* out, int heads, int key_dim,
+static void launch_latent(dim3 grid, hipStream_t s, const bf16* q, bf16* out, int heads, int key_dim,
                           int v_dim, const int32_t* positions, const int32_t* token_seq, const int32_t* tables,
                           int table_stride, const bf16* pool, int page_size, int num_pages, int window, int chunk,
                           float scale, float* partial, int nsplit) {
-  const size_t lds = static_cast<size_t>(32) * (KS * 32 + 16) * sizeof(uint16_t);
-  latent_attention_mfma_kernel<KS, DB><<<grid, waves * kWave, lds, s>>>(
+  const size_t lds = (static_cast<size_t>(32) * (KS * 32 + 32) + 64) * sizeof(uint16_t);
+  latent_attention_mfma_kernel<KS, DB><<<grid, kLatentWaves * kWave, lds, s>>>(
       q, out, heads, key_dim, v_dim, positions, token_seq, tables, table_stride, pool, page_size, num_pages, window,
       chunk, scale, partial, nsplit);
 }
@@ -240,11 +288,10 @@ extern "C" int shk_latent_attention_bf16(const void* q, void* out, int n, int he
   SHK_REQUIRE(reinterpret_cast<uintptr_t>(q) % 16 == 0 && reinterpret_cast<uintptr_t>(pool) % 16 == 0,
               "latent_attention_bf16: q and the pool must be 16-byte aligned");
   hipStream_t s = static_cast<hipStream_t>(stream);
-  const int waves = (heads + 15) / 16;
-  dim3 grid(n, nsplit);
+  dim3 grid(n, nsplit, (heads + 16 * kLatentWaves - 1) / (16 * kLatentWaves));
   const int ks = (key_dim + 31) / 32, db = (v_dim + 15) / 16;
 #define SHK_LATENT(KS, DB)                                                                                         \
-  launch_latent<KS, DB>(grid, waves, s, static_cast<const bf16*>(q), static_cast<bf16*>(out), heads, key_dim, v_dim, \
+  launch_latent<KS, DB>(grid, s, static_cast<const bf16*>(q), static_cast<bf16*>(out), heads, key_dim, v_dim, \
                         positions, token_seq, tables, table_stride, static_cast<const bf16*>(pool), page_size,      \
                         num_pages, window, chunk, scale, partial, nsplit)
   if (ks <= 4) { if (db <= 4) SHK_LATENT(4, 4); else SHK_LATENT(4, 8); }
