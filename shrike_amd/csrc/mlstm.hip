@@ -35,6 +35,20 @@ constexpr int kScanWaves = 8;   // wavefronts (tiles) per workgroup
 
 __host__ __device__ inline int scan_rpt(int dim) { return dim <= 64 ? 4 : dim <= 128 ? 8 : 16; }
 
+// Sum over the sixteen lanes that share a value column (lane = 4 * row group + column): the four
+// row groups of a 16-lane row by two rotations on the vector unit, then the four rows by two
+// exchanges through the LDS crossbar; every lane gets the sum, always in this order.
+template <int CTRL>
+__device__ __forceinline__ float scan_dpp(float v) {
+  return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xf, 0xf, true));
+}
+__device__ __forceinline__ float column_sum(float v) {
+  v += scan_dpp<0x124>(v);  // row_ror:4
+  v += scan_dpp<0x128>(v);  // row_ror:8
+  v += __shfl_xor(v, 16, kWave);
+  return v + __shfl_xor(v, 32, kWave);
+}
+
 __device__ __forceinline__ float log_sigmoid(float x) {
   return x >= 0.f ? -log1pf(expf(-x)) : x - log1pf(expf(x));
 }
@@ -136,11 +150,8 @@ __global__ void __launch_bounds__(kScanWaves* kWave)
           nq = fmaf(nv[i4 + u], qr[u], nq);
         }
       }
-#pragma unroll
-      for (int off = kCols; off < kWave; off <<= 1) {  // over the sixteen lanes of a column, in a fixed order
-        o += __shfl_xor(o, off, kWave);
-        nq += __shfl_xor(nq, off, kWave);
-      }
+      o = column_sum(o);  // over the sixteen lanes of a column, in a fixed order
+      nq = column_sum(nq);
       m = m_new;
       const float den = fmaxf(fabsf(nq), expf(-m)) + 1e-6f;
       if (rg == 0 && vcol < v_dim) out[static_cast<size_t>(t0 + tt) * heads * v_dim + head * v_dim + vcol] = o / den;
