@@ -245,11 +245,14 @@ int shk_latent_attention(const void* q, void* out, int dtype, int n, int heads, 
 // The same on the matrix units for bfloat16 (latent_mfma.hip), where
 // shk_latent_attention_supports_mfma says so.  nsplit > 1 shares every token's rows among nsplit
 // workgroups, whose results pass through `partial` (n * heads * nsplit * (v_dim + 2) floats).
+// tokens_per_group > 1 lets a workgroup serve up to that many (2 or 4) neighbouring tokens where
+// their heads leave wavefronts free (prompt portions; the result is the same).
 int shk_latent_attention_supports_mfma(int heads, int key_dim, int v_dim);
 int shk_latent_attention_bf16(const void* q, void* out, int n, int heads, int key_dim, int v_dim,
                               const int32_t* positions, const int32_t* token_seq, const int32_t* tables,
                               int table_stride, const void* pool, int page_size, int num_pages, int window,
-                              int chunk, float scale, float* partial, int nsplit, void* stream);
+                              int chunk, float scale, float* partial, int nsplit, int tokens_per_group,
+                              void* stream);
 
 // A batch of products of one shape: out_b[n, m] = a_b[n, k] @ w_b[m, k]^T for b < batch, with
 // a_b = a + b * a_batch (rows lda apart), w_b = w + b * w_batch (contiguous), out_b = out + b *

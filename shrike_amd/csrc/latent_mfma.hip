@@ -49,7 +49,8 @@ __global__ void __launch_bounds__(kLatentWaves* kWave)
                                  int v_dim, const int32_t* __restrict__ positions,
                                  const int32_t* __restrict__ token_seq, const int32_t* __restrict__ tables,
                                  int table_stride, const bf16* __restrict__ pool, int page_size, int num_pages,
-                                 int window, int chunk, float scale, float* __restrict__ partial, int nsplit) {
+                                 int window, int chunk, float scale, float* __restrict__ partial, int nsplit,
+                                 int n, int tpw) {
   // Rows in LDS: KS * 32 elements and 64 bytes of padding (consecutive rows start 16 banks apart: the
   // sixteen rows x four 16-byte pieces of a score operand cover the banks evenly), and every group of 8
   // rows is shifted by 32 bytes more (the four groups that a transposed value read touches at once,
@@ -59,14 +60,28 @@ __global__ void __launch_bounds__(kLatentWaves* kWave)
   // 16-byte pieces of a chunk that a thread stages: 32 rows of at most 4 KS pieces, 256 threads
   constexpr int kPieces = (32 * 4 * KS + kLatentWaves * kWave - 1) / (kLatentWaves * kWave);
   extern __shared__ __attribute__((aligned(16))) uint16_t rows[];  // [32][STRIDE]
-  const int t = blockIdx.x, z = blockIdx.y;
+  // A workgroup serves tpw tokens that follow each other in the step (1, 2 or 4; more than one only
+  // where a token's heads leave wavefronts free: wavefront w then serves token w / (4 / tpw)).  (A step
+  // lists a prompt's tokens in order and the last ones read the most rows: they start first, so that
+  // the launch ends with light workgroups and not with its heaviest.)
+  const int group = gridDim.x - 1 - blockIdx.x, z = blockIdx.y;
   const int tid = threadIdx.x, nthreads = blockDim.x;
   const int wave = tid / kWave, lane = tid % kWave, j = lane % 16, g = lane / 16;
+  const int wpt = kLatentWaves / tpw;  // wavefronts a token
+  const int t0 = group * tpw;
+  const int t_last = t0 + tpw - 1 < n - 1 ? t0 + tpw - 1 : n - 1;
+  const int t = t0 + wave / wpt < n ? t0 + wave / wpt : t_last;  // (a wavefront past the step's end: idle below)
+  const bool has_token = t0 + wave / wpt < n;
   const int pos = positions[t];
   const int lo = first_key(pos, window, chunk);
-  const int32_t* table = tables + static_cast<size_t>(token_seq[t]) * table_stride;
-  const int head = (blockIdx.z * kLatentWaves + wave) * 16 + j;  // (more than 64 heads: several workgroups a token)
-  const bool col_ok = head < heads;
+  const int head = (blockIdx.z * kLatentWaves + wave % wpt) * 16 + j;  // (more than 64 heads: several workgroups a token)
+  const bool col_ok = has_token && head < heads;
+  // Tokens of one sequence share what is staged (their rows are the same but for the newest); where a
+  // workgroup's tokens belong to several sequences (single tokens of a batch, a portion's end) it
+  // takes them one after the other.
+  bool same = true;
+  for (int i = t0 + 1; i <= t_last; ++i) same = same && token_seq[i] == token_seq[t0];
+  const int passes = same ? 1 : t_last - t0 + 1;
 
   // the queries of this wavefront's heads as B operands: head j, elements 32 ks + 8 g ..
   LFrag qf[KS];
@@ -81,11 +96,6 @@ __global__ void __launch_bounds__(kLatentWaves* kWave)
   for (int i = tid; i < (32 * STRIDE + 64) / 8; i += nthreads) reinterpret_cast<uint4*>(rows)[i] = make_uint4(0, 0, 0, 0);
   __syncthreads();
 
-  const int key_begin = lo & ~31;
-  const int nchunks = (pos - key_begin) / 32 + 1;
-  const int per_split = (nchunks + nsplit - 1) / nsplit;
-  const int c_first = z * per_split;
-  const int c_end = c_first + per_split < nchunks ? c_first + per_split : nchunks;
   const int npieces = key_dim / 8;
   const float scale2 = scale * 1.4426950408889634f;
 
@@ -109,13 +119,24 @@ __global__ void __launch_bounds__(kLatentWaves* kWave)
     piece_lds[u] = at(piece_row[u] < 0 ? 0 : piece_row[u]) + piece_col[u];
   }
   const int page_shift = (page_size & (page_size - 1)) == 0 ? __ffs(page_size) - 1 : -1;
+  for (int pass = 0; pass < passes; ++pass) {
+  // the tokens of this pass: all of the workgroup's, or its pass-th; positions rise along a portion
+  const int ta = same ? t0 : t0 + pass, tb = same ? t_last : t0 + pass;
+  const int stage_hi = positions[tb], stage_lo = first_key(positions[ta], window, chunk);
+  const int32_t* table = tables + static_cast<size_t>(token_seq[ta]) * table_stride;
+  const bool mine = has_token && t >= ta && t <= tb && head - j < heads;  // this wavefront multiplies in this pass
+  const int key_begin = stage_lo & ~31;
+  const int nchunks = (stage_hi - key_begin) / 32 + 1;
+  const int per_split = (nchunks + nsplit - 1) / nsplit;
+  const int c_first = z * per_split;
+  const int c_end = c_first + per_split < nchunks ? c_first + per_split : nchunks;
   auto fetch = [&](int c) {
     const int kb = key_begin + c * 32;
 #pragma unroll
     for (int u = 0; u < kPieces; ++u) {
       const int key = kb + piece_row[u];
       staged[u] = make_uint4(0, 0, 0, 0);
-      if (piece_row[u] >= 0 && key >= lo && key <= pos) {
+      if (piece_row[u] >= 0 && key >= stage_lo && key <= stage_hi) {
         const int entry = page_shift >= 0 ? key >> page_shift : key / page_size;
         const int slot = page_shift >= 0 ? key & (page_size - 1) : key % page_size;
         const int page = table[entry];
@@ -136,7 +157,7 @@ __global__ void __launch_bounds__(kLatentWaves* kWave)
     put();
     __syncthreads();
     if (c + 1 < c_end) fetch(c + 1);  // (the same for every thread of the workgroup)
-    if (head - j >= heads) {  // a wavefront that only helps to stage
+    if (!mine) {  // a wavefront that only helps to stage in this pass
       __syncthreads();
       continue;
     }
@@ -179,7 +200,7 @@ __global__ void __launch_bounds__(kLatentWaves* kWave)
 #pragma unroll
       for (int db = 0; db < DB; ++db) o[db] *= alpha;
     }
-    const uint16_t* mine = rows + at(8 * g) + j;  // rows 8 g .. 8 g + 7 lie STRIDE apart
+    const uint16_t* vrows = rows + at(8 * g) + j;  // rows 8 g .. 8 g + 7 lie STRIDE apart
 #pragma unroll
     for (int db = 0; db < DB; ++db) {
       // (packed by hand into a native vector: halves written one by one into a union's array
@@ -187,12 +208,13 @@ __global__ void __launch_bounds__(kLatentWaves* kWave)
       lu32x4 vw;
 #pragma unroll
       for (int e2 = 0; e2 < 4; ++e2)
-        vw[e2] = static_cast<uint32_t>(mine[(2 * e2) * STRIDE + db * 16]) |
-                 (static_cast<uint32_t>(mine[(2 * e2 + 1) * STRIDE + db * 16]) << 16);
+        vw[e2] = static_cast<uint32_t>(vrows[(2 * e2) * STRIDE + db * 16]) |
+                 (static_cast<uint32_t>(vrows[(2 * e2 + 1) * STRIDE + db * 16]) << 16);
       o[db] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(lbf16x8, vw), pf.v, o[db], 0, 0, 0);
     }
     __syncthreads();  // the next chunk overwrites the rows
   }
+  }  // passes
   l = quad_lanes_sum(l);
   if (!col_ok) return;  // (no barrier follows)
 
@@ -210,7 +232,7 @@ __global__ void __launch_bounds__(kLatentWaves* kWave)
     return;
   }
   // a share's result: O [row][share][v_dim], then (maximum, sum) [row][share][2]
-  const size_t all_rows = static_cast<size_t>(gridDim.x) * heads;  // (gridDim.x: the step's tokens)
+  const size_t all_rows = static_cast<size_t>(n) * heads;
   float* dst = partial + (row * nsplit + z) * v_dim;
 #pragma unroll
   for (int db = 0; db < DB; ++db)
@@ -254,11 +276,11 @@ template <int KS, int DB>
 static void launch_latent(dim3 grid, hipStream_t s, const bf16* q, bf16* out, int heads, int key_dim,
                           int v_dim, const int32_t* positions, const int32_t* token_seq, const int32_t* tables,
                           int table_stride, const bf16* pool, int page_size, int num_pages, int window, int chunk,
-                          float scale, float* partial, int nsplit) {
+                          float scale, float* partial, int nsplit, int n, int tpw) {
   const size_t lds = (static_cast<size_t>(32) * (KS * 32 + 32) + 64) * sizeof(uint16_t);
   latent_attention_mfma_kernel<KS, DB><<<grid, kLatentWaves * kWave, lds, s>>>(
       q, out, heads, key_dim, v_dim, positions, token_seq, tables, table_stride, pool, page_size, num_pages, window,
-      chunk, scale, partial, nsplit);
+      chunk, scale, partial, nsplit, n, tpw);
 }
 
 }  // namespace shk
@@ -275,10 +297,12 @@ extern "C" int shk_latent_attention_supports_mfma(int heads, int key_dim, int v_
 extern "C" int shk_latent_attention_bf16(const void* q, void* out, int n, int heads, int key_dim, int v_dim,
                                          const int32_t* positions, const int32_t* token_seq, const int32_t* tables,
                                          int table_stride, const void* pool, int page_size, int num_pages, int window,
-                                         int chunk, float scale, float* partial, int nsplit, void* stream) {
+                                         int chunk, float scale, float* partial, int nsplit, int tokens_per_group,
+                                         void* stream) {
   SHK_REQUIRE(shk_latent_attention_supports_mfma(heads, key_dim, v_dim),
               "latent_attention_bf16: %d heads over rows of %d with values of %d are not served", heads, key_dim, v_dim);
-  SHK_REQUIRE(n >= 0 && n <= 1 << 30 && nsplit >= 1 && nsplit <= 64, "latent_attention_bf16: bad sizes n=%d nsplit=%d", n, nsplit);
+  SHK_REQUIRE(n >= 0 && n <= 1 << 30 && nsplit >= 1 && nsplit <= 64 && tokens_per_group >= 1,
+              "latent_attention_bf16: bad sizes n=%d nsplit=%d tokens_per_group=%d", n, nsplit, tokens_per_group);
   SHK_REQUIRE(page_size > 0 && num_pages > 0 && table_stride > 0,
               "latent_attention_bf16: bad cache sizes page_size=%d num_pages=%d table_stride=%d", page_size, num_pages,
               table_stride);
@@ -288,12 +312,16 @@ extern "C" int shk_latent_attention_bf16(const void* q, void* out, int n, int he
   SHK_REQUIRE(reinterpret_cast<uintptr_t>(q) % 16 == 0 && reinterpret_cast<uintptr_t>(pool) % 16 == 0,
               "latent_attention_bf16: q and the pool must be 16-byte aligned");
   hipStream_t s = static_cast<hipStream_t>(stream);
-  dim3 grid(n, nsplit, (heads + 16 * kLatentWaves - 1) / (16 * kLatentWaves));
+  // tokens a workgroup: as many as its four wavefronts hold (16 heads each), if the caller allows
+  int tpw = 1;
+  if (tokens_per_group > 1 && heads <= 32) tpw = heads <= 16 ? 4 : 2;
+  if (tpw > tokens_per_group) tpw = tokens_per_group >= 2 ? 2 : 1;
+  dim3 grid((n + tpw - 1) / tpw, nsplit, (heads + 16 * kLatentWaves - 1) / (16 * kLatentWaves));
   const int ks = (key_dim + 31) / 32, db = (v_dim + 15) / 16;
 #define SHK_LATENT(KS, DB)                                                                                         \
   launch_latent<KS, DB>(grid, s, static_cast<const bf16*>(q), static_cast<bf16*>(out), heads, key_dim, v_dim, \
                         positions, token_seq, tables, table_stride, static_cast<const bf16*>(pool), page_size,      \
-                        num_pages, window, chunk, scale, partial, nsplit)
+                        num_pages, window, chunk, scale, partial, nsplit, n, tpw)
   if (ks <= 4) { if (db <= 4) SHK_LATENT(4, 4); else SHK_LATENT(4, 8); }
   else if (ks <= 8) { if (db <= 8) SHK_LATENT(8, 8); else SHK_LATENT(8, 16); }
   else if (ks <= 16) { if (db <= 16) SHK_LATENT(16, 16); else SHK_LATENT(16, 32); }

@@ -50,7 +50,7 @@ _SIGNATURES = {
     "shk_rotate_heads": [_P, _I, _I, _I, _P, _I, _I, _I, _I, _I, _I, _I, _P, _P, _P],
     "shk_latent_attention": [_P, _P, _I, _I, _I, _I, _I, _P, _P, _P, _I, _P, _I, _I, _I, _I, _F, _P],
     "shk_latent_attention_supports_mfma": [_I, _I, _I],
-    "shk_latent_attention_bf16": [_P, _P, _I, _I, _I, _I, _P, _P, _P, _I, _P, _I, _I, _I, _I, _F, _P, _I, _P],
+    "shk_latent_attention_bf16": [_P, _P, _I, _I, _I, _I, _P, _P, _P, _I, _P, _I, _I, _I, _I, _F, _P, _I, _I, _P],
     "shk_gemm_batched": [_P, _P, _P, _I, _I, _I, _I, _I, _I, c_longlong, c_longlong, c_longlong, _I, _P],
     "shk_mlstm_scan": [_P, _I, _I, _I, _I, _I, _I, _P, _P, _F, _F, _I, _I, _I, _I, _P, _P, _P, _P, c_longlong, _P, _P],
     "shk_headnorm_gate": [_P, _P, _I, _P, _F, _P, _I, _I, _I, _I, _P],

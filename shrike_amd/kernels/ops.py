@@ -582,9 +582,10 @@ def latent_attention_supports_mfma(heads: int, key_dim: int, v_dim: int) -> bool
 
 
 def latent_attention_mfma(q, out, heads, key_dim, v_dim, positions, token_seq, tables, pool, page_size, window,
-                          scale, chunk=None, partial=None, nsplit: int = 1) -> None:
+                          scale, chunk=None, partial=None, nsplit: int = 1, tokens_per_group: int = 1) -> None:
     """latent_attention on the matrix units (bfloat16).  nsplit > 1 shares each token's rows among
-    that many workgroups; partial: float32 scratch of n * heads * nsplit * (v_dim + 2)."""
+    that many workgroups; partial: float32 scratch of n * heads * nsplit * (v_dim + 2).
+    tokens_per_group: up to how many neighbouring tokens a workgroup may serve (prompt portions)."""
     n = q.shape[0]
     if q.dtype != torch.bfloat16 or out.dtype != torch.bfloat16:
         raise KernelError("latent_attention_mfma: bfloat16 only")
@@ -604,7 +605,8 @@ def latent_attention_mfma(q, out, heads, key_dim, v_dim, positions, token_seq, t
         _dev(q, "q"), _dev(out, "out"), n, heads, key_dim, v_dim, _dev(positions, "positions", torch.int32),
         _dev(token_seq, "token_seq", torch.int32), _dev(tables, "tables", torch.int32), tables.shape[1],
         _dev(pool, "pool"), page_size, pool.shape[0], int(window or 0), int(chunk or 0), float(scale),
-        _dev(partial, "partial", torch.float32) if nsplit > 1 else None, int(nsplit), _stream()))
+        _dev(partial, "partial", torch.float32) if nsplit > 1 else None, int(nsplit), int(tokens_per_group),
+        _stream()))
 
 
 def gemm_batched(a, w, out, batch: int, a_step: int, out_step: int) -> None:

@@ -92,8 +92,10 @@ class LatentAttention(Mixer):
             while keys < reach:
                 keys *= 2
             nsplit = max(1, min(2 * compute_units() // tokens, keys // 128, 64))
-        shape.notes[key] = nsplit
-        shape.launch_key.append((key, nsplit))
+        # a step with prompt portions: neighbouring tokens may share a workgroup (and what it stages)
+        group = 1 if shape.num_decode == shape.num_seqs else 4
+        shape.notes[key] = (nsplit, group)
+        shape.launch_key.append((key, nsplit, group))
 
     def load(self, tensors, runtime):
         s = self.spec
@@ -141,13 +143,13 @@ class LatentAttention(Mixer):
                          ctx.positions)
         mixed = ctx.buffer("latent_mixed", (n, H * s.kv_rank), ctx.dtype)
         if self.mfma:
-            nsplit = ctx.notes[("latent_attention", H, s.kv_rank, s.rot_dim, s.window, s.chunk)]
+            nsplit, group = ctx.notes[("latent_attention", H, s.kv_rank, s.rot_dim, s.window, s.chunk)]
             partial = None
             if nsplit > 1:
                 partial = ctx.buffer("latent_partial", (n * H * nsplit * (s.kv_rank + 2),), torch.float32)
             ops.latent_attention_mfma(folded, mixed, H, key_dim, s.kv_rank, ctx.positions, ctx.token_seq, tables,
                                       cache.pools["latent"], cache.page_size, s.window, s.scale, chunk=s.chunk,
-                                      partial=partial, nsplit=nsplit)
+                                      partial=partial, nsplit=nsplit, tokens_per_group=group)
         else:
             ops.latent_attention(folded, mixed, H, key_dim, s.kv_rank, ctx.positions, ctx.token_seq, tables,
                                  cache.pools["latent"], cache.page_size, s.window, s.scale, chunk=s.chunk)

@@ -307,13 +307,16 @@ def test_latent_attention_at_the_windows_edges(ops, dtype, heads, key_dim, v_dim
     close(out.view(n, heads, v_dim), want, dtype)
     if dtype == torch.bfloat16 and ops.latent_attention_supports_mfma(heads, key_dim, v_dim):
         # the same on the matrix units, each token's rows taken by one workgroup and shared among three
-        for nsplit in (1, 3):
+        # ... and with up to four neighbouring tokens a workgroup (the first workgroups hold single tokens
+        # of different sequences, one holds a portion's first tokens beside one of them)
+        for nsplit, group in ((1, 1), (3, 1), (1, 4), (2, 2)):
             again = torch.full((n, heads * v_dim), float("nan"), dtype=dtype, device="cuda")
             partial = torch.full((n * heads * nsplit * (v_dim + 2),), float("nan"), device="cuda")
             ops.latent_attention_mfma(dev(q.reshape(n, heads * key_dim)), again, heads, key_dim, v_dim, positions, token_seq,
-                                      dev(tables), pool, page_size, window, scale, partial=partial, nsplit=nsplit)
+                                      dev(tables), pool, page_size, window, scale, partial=partial, nsplit=nsplit,
+                                      tokens_per_group=group)
             assert torch.isfinite(again).all(), f"{nsplit} shares: a row outside the window or the pages was read"
-            close(again.view(n, heads, v_dim), want, dtype, f"matrix units, {nsplit} shares")
+            close(again.view(n, heads, v_dim), want, dtype, f"matrix units, {nsplit} shares, {group} tokens a workgroup")
     assert window >= 300 or (any(inside for _, inside in marks) and any(not inside for _, inside in marks))
 
 
