@@ -420,7 +420,7 @@ def minilorn_like(qcfg, window: int, pattern: str):
     up64 = lambda x: max(64, -(-int(x) // 64) * 64)  # noqa: E731
     mixers = {
         "a": ("attention", SinkAttention(heads=H, kv_heads=qcfg.num_key_value_heads, dim=d, vdim=d, scale=d**-0.5,
-                                         softcap=50.0, q_temp=(0.5, 128))),
+                                         softcap=30.0, q_temp=(0.25, 256))),
         "l": ("latent_attention", LatentAttention(heads=H, dim=d, rot_dim=d // 2, vdim=d, q_rank=up64(3 * h / 8),
                                                    kv_rank=up64(h / 8), scale=(1.5 * d) ** -0.5, rot_base=10000.0,
                                                    window=window, rot_dims=d // 2)),
