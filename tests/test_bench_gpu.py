@@ -40,3 +40,21 @@ def test_products_mode_times_every_product_of_a_layer_both_ways():
     assert set(got) == {f"{name}_n{n}" for n in (8, 200) for name in ("qkv", "o", "gate_up", "down")} | {"lm_head_n8"}
     for entry in got.values():
         assert entry["own_us"] > 0 and entry["library_us"] > 0 and entry["k_shares"] >= 1
+
+
+def test_the_second_design_of_the_comparison_is_built_from_the_first_ones_sizes_and_decodes():
+    """bench.py --minilorn: a Minilorn with a Qwen2 configuration's width, heads, feed-forward width and
+    number of layers, every mixer in the pattern's order; it takes prompts in and decodes like the other."""
+    import shrike_amd.models  # noqa: F401
+    from shrike_amd.models import minilorn
+    from shrike_amd.models.qwen2 import Qwen2Config
+
+    qcfg = Qwen2Config.from_dict(dict(CONFIGS["B"], torch_dtype="bfloat16"))
+    mcfg, sizes = bench.minilorn_like(qcfg, window=48, pattern="lma")
+    assert [layer.type for layer in mcfg.layers][:3] == ["latent_attention", "mlstm", "attention"][: len(mcfg.layers)]
+    assert len(mcfg.layers) == qcfg.num_hidden_layers and mcfg.width == qcfg.hidden_size
+    assert all(layer.ff == qcfg.intermediate_size for layer in mcfg.layers)
+    assert sizes.layer_elements > 2 * qcfg.hidden_size * qcfg.intermediate_size and sizes.kv_elements_per_token > 0
+    engine = bench.make_engine(sizes, minilorn.build_spec(mcfg), 4, seed=1)
+    run = bench.run_decode(engine, sizes, 4, steps=10, warmup=2, seed=5, prompt_len=70)
+    assert run["context_end"] - run["context_start"] == 10 and run["tok_s"] > 0
