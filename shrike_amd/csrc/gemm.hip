@@ -162,7 +162,8 @@ extern "C" int shk_gemm_batched(const void* a, const void* w, void* out, int n, 
   SHK_REQUIRE(a && w && out, "gemm_batched: null pointer");
   SHK_REQUIRE((n + kTM - 1) / kTM <= 65535, "gemm_batched: too many rows (%d)", n);
   hipStream_t s = static_cast<hipStream_t>(stream);
-  if (n <= 2 * kSkinnyRows) {
+  // (float32 keeps one order of summation whatever the number of rows: the tiled kernel's ascending k)
+  if (n <= 2 * kSkinnyRows && dtype == kBF16) {
     dim3 grid((m + 3) / 4, batch);
     if (dtype == kF32)
       gemm_batched_skinny_kernel<float><<<grid, 256, 0, s>>>(static_cast<const float*>(a), static_cast<const float*>(w),
