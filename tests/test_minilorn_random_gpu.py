@@ -88,8 +88,8 @@ def test_a_random_configuration_in_four_cuttings(seed, dtype, tmp_path):
         err = np.abs(row.astype(np.float64) - want[name][pos]).max() / np.abs(want[name]).max()
         if dtype == "float32":
             assert err <= 1e-4, f"seed {seed} ({cfg}): {rid} position {pos}: rel err {err:.3e}"
-            # the cuttings agree with each other more closely still
-            assert np.abs(row - got[(f"w_{name}", pos)]).max() / np.abs(want[name]).max() <= 1e-5
+            # every float32 kernel sums in one order whatever else is in the step: the same bits in every cutting
+            assert np.array_equal(row, got[(f"w_{name}", pos)]), f"seed {seed}: {rid} position {pos} depends on the cutting"
         elif err > 1.5e-2:
             over.append((name, pos, err))
     # bfloat16: a few positions where a memory's readout is nearly nothing or capped scores are steep
