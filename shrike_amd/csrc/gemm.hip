@@ -148,6 +148,60 @@ extern "C" int shk_gemm(const void* a, const void* w, const float* bias, void* o
   return 0;
 }
 
+// The same batch on the matrix units for bfloat16: both operands are row-major with k innermost, which
+// is the operand layout of v_mfma_f32_16x16x32_bf16 as it stands (a lane's 8 consecutive k of one row
+// are one 16-byte load), so nothing passes through LDS.  A wavefront forms 16 rows x 64 features (four
+// tiles that share the rows' operand); a workgroup of four wavefronts 64 x 64.  k in multiples of 8
+// and 16-byte aligned rows; a wavefront's result does not depend on what else is in the step.
+typedef __bf16 gbf16x8 __attribute__((ext_vector_type(8)));
+typedef float gf32x4 __attribute__((ext_vector_type(4)));
+
+__global__ void __launch_bounds__(256)
+    gemm_batched_mfma_kernel(const bf16* __restrict__ a, const bf16* __restrict__ w, bf16* __restrict__ out, int n,
+                             int m, int k, int lda, int ldo, long long a_batch, long long w_batch,
+                             long long out_batch) {
+  const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
+  const int i = lane % 16, kg = lane / 16;
+  const int b = blockIdx.z;
+  const int row = (blockIdx.y * 4 + wave) * 16 + i;  // the row of a whose operand this lane loads
+  const int col0 = blockIdx.x * 64;
+  const bf16* ar = a + b * a_batch + static_cast<size_t>(row < n ? row : 0) * lda + kg * 8;
+  const bf16* wr[4];
+#pragma unroll
+  for (int t = 0; t < 4; ++t) {
+    const int c = col0 + t * 16 + i;  // the feature whose weights this lane loads for tile t
+    wr[t] = w + b * w_batch + static_cast<size_t>(c < m ? c : 0) * k + kg * 8;
+  }
+  gf32x4 acc[4];
+#pragma unroll
+  for (int t = 0; t < 4; ++t) acc[t] = gf32x4{0.f, 0.f, 0.f, 0.f};
+  for (int k0 = 0; k0 < k; k0 += 32) {
+    const bool have = k0 + kg * 8 < k;  // (k is a multiple of 8: a piece is whole or absent)
+    uint4 av = make_uint4(0, 0, 0, 0), wv[4];
+    if (have && row < n) av = *reinterpret_cast<const uint4*>(ar + k0);
+#pragma unroll
+    for (int t = 0; t < 4; ++t) {
+      wv[t] = make_uint4(0, 0, 0, 0);
+      if (have && col0 + t * 16 + i < m) wv[t] = *reinterpret_cast<const uint4*>(wr[t] + k0);
+    }
+#pragma unroll
+    for (int t = 0; t < 4; ++t)
+      acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(gbf16x8, wv[t]), __builtin_bit_cast(gbf16x8, av),
+                                                       acc[t], 0, 0, 0);
+  }
+  // the products were formed transposed (features as rows): this lane holds features 4 kg + r of tile t for row i
+  const int orow = (blockIdx.y * 4 + wave) * 16 + i;
+  if (orow >= n) return;
+  bf16* dst = out + b * out_batch + static_cast<size_t>(orow) * ldo;
+#pragma unroll
+  for (int t = 0; t < 4; ++t)
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      const int c = col0 + t * 16 + 4 * kg + r;
+      if (c < m) dst[c] = from_float<bf16>(acc[t][r]);
+    }
+}
+
 // A batch of products of one shape (one per head, say): product b reads a + b * a_batch
 // (rows lda apart), w + b * w_batch ([m, k] contiguous) and writes out + b * out_batch.
 extern "C" int shk_gemm_batched(const void* a, const void* w, void* out, int n, int m, int k, int lda,
@@ -162,8 +216,13 @@ extern "C" int shk_gemm_batched(const void* a, const void* w, void* out, int n, 
   SHK_REQUIRE(a && w && out, "gemm_batched: null pointer");
   SHK_REQUIRE((n + kTM - 1) / kTM <= 65535, "gemm_batched: too many rows (%d)", n);
   hipStream_t s = static_cast<hipStream_t>(stream);
-  // (float32 keeps one order of summation whatever the number of rows: the tiled kernel's ascending k)
-  if (n <= 2 * kSkinnyRows && dtype == kBF16) {
+  if (dtype == kBF16 && k % 8 == 0 && lda % 8 == 0 && a_batch % 8 == 0 && reinterpret_cast<uintptr_t>(a) % 16 == 0 &&
+      reinterpret_cast<uintptr_t>(w) % 16 == 0 && (n + 63) / 64 <= 65535) {
+    dim3 grid((m + 63) / 64, (n + 63) / 64, batch);
+    gemm_batched_mfma_kernel<<<grid, 256, 0, s>>>(static_cast<const bf16*>(a), static_cast<const bf16*>(w),
+                                                  static_cast<bf16*>(out), n, m, k, lda, ldo, a_batch, w_batch, out_batch);
+  } else if (n <= 2 * kSkinnyRows && dtype == kBF16) {
+    // (float32 keeps one order of summation whatever the number of rows: the tiled kernel's ascending k)
     dim3 grid((m + 3) / 4, batch);
     if (dtype == kF32)
       gemm_batched_skinny_kernel<float><<<grid, 256, 0, s>>>(static_cast<const float*>(a), static_cast<const float*>(w),

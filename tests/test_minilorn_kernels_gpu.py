@@ -322,18 +322,21 @@ def test_latent_attention_at_the_windows_edges(ops, dtype, heads, key_dim, v_dim
 
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("n, batch, m, k", [(1, 6, 96, 40), (70, 3, 10, 24), (5, 2, 65, 130), (32, 4, 7, 300), (33, 2, 64, 64),
-                                            (17, 28, 448, 128)])
+                                            (17, 28, 448, 128), (200, 3, 130, 72), (8, 5, 16, 8)])
 def test_batched_product(ops, dtype, n, batch, m, k):
+    """Slices of a that are 16-byte aligned (what bfloat16 then runs on the matrix units) and slices
+    that are not (the general kernels)."""
     torch.manual_seed(7)
-    a_step, out_step = k + 3, m + 5
-    a = torch.randn(n, batch * a_step).to(dtype)
-    w = (torch.randn(batch, m, k) / k**0.5).to(dtype)
-    out = torch.zeros(n, batch * out_step, dtype=dtype, device="cuda")
-    ops.gemm_batched(dev(a), dev(w), out, batch, a_step, out_step)
-    for b in range(batch):
-        want = a[:, b * a_step : b * a_step + k].double() @ w[b].double().T
-        close(out[:, b * out_step : b * out_step + m], want, dtype, f"product {b}")
-        assert float(out[:, b * out_step + m : (b + 1) * out_step].abs().max()) == 0.0
+    for a_pad in (3, 8):
+        a_step, out_step = k + a_pad, m + 5
+        a = torch.randn(n, batch * a_step).to(dtype)
+        w = (torch.randn(batch, m, k) / k**0.5).to(dtype)
+        out = torch.zeros(n, batch * out_step, dtype=dtype, device="cuda")
+        ops.gemm_batched(dev(a), dev(w), out, batch, a_step, out_step)
+        for b in range(batch):
+            want = a[:, b * a_step : b * a_step + k].double() @ w[b].double().T
+            close(out[:, b * out_step : b * out_step + m], want, dtype, f"product {b}, slices {a_step} apart")
+            assert float(out[:, b * out_step + m : (b + 1) * out_step].abs().max()) == 0.0
 
 
 # ------------------------------------------------------------------ matrix memory
